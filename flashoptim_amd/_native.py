@@ -1,0 +1,110 @@
+"""ctypes binding of libflashoptim_hip.so (C ABI declared in include/flashoptim_hip.h).
+
+The library is the only implementation of the step math in this package: if it cannot be loaded the
+package raises, it never falls back to PyTorch ops.  Calls release the GIL (plain ``ctypes.CDLL``), take
+raw ``data_ptr()`` values and the current HIP stream, and return immediately after enqueueing.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from typing import Optional
+
+import torch
+
+_LIB_NAME = "libflashoptim_hip.so"
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", _LIB_NAME)
+
+DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+TILE_ELEMS = 4096
+
+
+class FoTensorDesc(ctypes.Structure):
+    """Mirror of ``fo_tensor_desc``."""
+
+    _fields_ = [
+        ("param", ctypes.c_void_p),
+        ("grad", ctypes.c_void_p),
+        ("ecc", ctypes.c_void_p),
+        ("mom", ctypes.c_void_p),
+        ("mom_scales", ctypes.c_void_p),
+        ("var", ctypes.c_void_p),
+        ("var_scales", ctypes.c_void_p),
+        ("n", ctypes.c_int64),
+    ]
+
+
+class FoChunk(ctypes.Structure):
+    """Mirror of ``fo_chunk``."""
+
+    _fields_ = [
+        ("tensor", ctypes.c_int32),
+        ("first_tile", ctypes.c_int32),
+        ("n_tiles", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+_lock = threading.Lock()
+_lib: Optional[ctypes.CDLL] = None
+
+# name -> (restype, argtypes); kept in one table so a test can check it against the header
+_vp, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+SIGNATURES = {
+    "fo_version": (_i32, []),
+    "fo_last_error": (ctypes.c_char_p, []),
+    "fo_device_compute_units": (_i32, [_i32]),
+    "fo_adam_step": (_i32, [_vp] * 7 + [_i64, _i32, _i32, _i32] + [_f32] * 5 + [_i32, _i32, _vp]),
+    "fo_momentum_step": (_i32, [_vp] * 5 + [_i64, _i32, _i32, _i32] + [_f32] * 4 + [_i32, _i32, _i32, _vp]),
+    "fo_sgd_plain_step": (_i32, [_vp] * 3 + [_i64, _i32, _i32, _f32, _f32, _i32, _vp]),
+    "fo_count_chunks": (_i64, [_vp, _i64, _i32]),
+    "fo_build_chunks": (_i64, [_vp, _i64, _i32, _vp, _i64]),
+    "fo_multi_adam_step": (_i32, [_vp, _i64, _vp, _i64, _i32, _i32, _i32] + [_f32] * 5 + [_i32, _i32, _vp]),
+    "fo_multi_momentum_step": (_i32, [_vp, _i64, _vp, _i64, _i32, _i32, _i32] + [_f32] * 4 + [_i32, _i32, _i32, _vp]),
+    "fo_quantize": (_i32, [_vp, _i32, _vp, _vp, _i64, _i32, _i32, _i32, _vp]),
+    "fo_dequantize": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp]),
+    "fo_ecc_join": (_i32, [_vp, _i32, _vp, _i32, _vp, _i64, _vp]),
+    "fo_ecc_split": (_i32, [_vp, _vp, _i32, _vp, _i32, _i64, _vp]),
+    "fo_copy_bytes": (_i32, [_vp, _vp, _i64, _vp]),
+}
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    """Load the HIP library once; raise loudly when it has not been built."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.exists(_LIB_PATH):
+                    raise RuntimeError(
+                        f"{_LIB_PATH} is missing: flashoptim_amd has no implementation without its HIP "
+                        "library. Build it with `make -C flashoptim_amd/csrc` (or __graft_entry__.build())."
+                    )
+                handle = ctypes.CDLL(_LIB_PATH)
+                for name, (restype, argtypes) in SIGNATURES.items():
+                    fn = getattr(handle, name)
+                    fn.restype = restype
+                    fn.argtypes = argtypes
+                _lib = handle
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    """Translate a non-zero native return code into RuntimeError with the library's message."""
+    if rc != 0:
+        msg = lib().fo_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what} failed (code {rc}): {msg}")
+
+
+def current_stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()

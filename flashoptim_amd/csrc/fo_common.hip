@@ -1,0 +1,116 @@
+// Library-wide pieces of libflashoptim_hip.so: error text, device queries, the host-side chunk-table builder
+// of the multi-tensor launcher and the calibration copy kernel.
+#include "fo_device.h"
+#include "fo_host.h"
+#include "../../include/flashoptim_hip.h"
+
+#include <cstdarg>
+#include <cstdio>
+
+namespace fo {
+
+// plain copy with the same access shape; calibrates byte counters and shows the attainable streaming rate
+__global__ __launch_bounds__(kBlockThreads) void copy_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, int64_t n_vec) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < n_vec; i += (int64_t)gridDim.x * kBlockThreads)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+
+}  // namespace fo
+
+namespace fo_host {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return 0;
+    snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(e));
+    return (int)e;
+}
+
+const char* last_error() { return g_err; }
+
+int compute_units() {
+    static thread_local int cached_dev = -1, cached_cus = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (dev != cached_dev) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cached_dev = dev; cached_cus = cus;
+    }
+    return cached_cus;
+}
+
+}  // namespace fo_host
+
+using namespace fo_host;
+
+extern "C" {
+
+int fo_version(void) { return 100; }
+const char* fo_last_error(void) { return last_error(); }
+
+int fo_device_compute_units(int device) {
+    int cus = 0;
+    hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+    if (e != hipSuccess) { check_hip(e, "hipDeviceGetAttribute"); return FO_ERR_NO_DEVICE; }
+    return cus;
+}
+
+int64_t fo_count_chunks(const int64_t* numels, int64_t n_tensors, int tiles_per_chunk) {
+    if (!numels || n_tensors < 0) return fail(FO_ERR_INVALID_ARGUMENT, "bad tensor length array");
+    const int64_t tpc = tiles_per_chunk > 0 ? tiles_per_chunk : kDefaultTilesPerChunk;
+    int64_t total = 0;
+    for (int64_t i = 0; i < n_tensors; ++i) {
+        if (numels[i] < 0) return fail(FO_ERR_INVALID_ARGUMENT, "tensor %lld has negative length", (long long)i);
+        const int64_t tiles = (numels[i] + fo::kTileElems - 1) / fo::kTileElems;
+        total += (tiles + tpc - 1) / tpc;
+    }
+    return total;
+}
+
+int64_t fo_build_chunks(const int64_t* numels, int64_t n_tensors, int tiles_per_chunk, fo_chunk* out, int64_t capacity) {
+    const int64_t need = fo_count_chunks(numels, n_tensors, tiles_per_chunk);
+    if (need < 0) return need;
+    if (!out || capacity < need) return fail(FO_ERR_INVALID_ARGUMENT, "chunk buffer too small (%lld < %lld)", (long long)capacity, (long long)need);
+    if (n_tensors > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "too many tensors");
+    const int64_t tpc = tiles_per_chunk > 0 ? tiles_per_chunk : kDefaultTilesPerChunk;
+    int64_t c = 0;
+    for (int64_t i = 0; i < n_tensors; ++i) {
+        const int64_t tiles = (numels[i] + fo::kTileElems - 1) / fo::kTileElems;
+        if (tiles > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "tensor %lld too large", (long long)i);
+        for (int64_t t0 = 0; t0 < tiles; t0 += tpc) {
+            out[c].tensor = (int32_t)i;
+            out[c].first_tile = (int32_t)t0;
+            out[c].n_tiles = (int32_t)((tiles - t0) < tpc ? (tiles - t0) : tpc);
+            out[c].reserved = 0;
+            ++c;
+        }
+    }
+    return c;
+}
+
+int fo_copy_bytes(void* dst, const void* src, int64_t n_bytes, void* stream) {
+    if (n_bytes < 0 || (n_bytes & 15)) return fail(FO_ERR_INVALID_ARGUMENT, "n_bytes must be a non-negative multiple of 16");
+    if (n_bytes == 0) return 0;
+    if (!dst || !src || (((uintptr_t)dst | (uintptr_t)src) & 15)) return fail(FO_ERR_INVALID_ARGUMENT, "copy pointers must be 16-byte aligned");
+    const int cus = compute_units();
+    if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
+    const int64_t n_vec = n_bytes / 16;
+    const int64_t want = (n_vec + fo::kBlockThreads - 1) / fo::kBlockThreads;
+    const int64_t cap = (int64_t)cus * kBlocksPerCu * 2;
+    hipLaunchKernelGGL(fo::copy_kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(fo::kBlockThreads), 0, (hipStream_t)stream,
+                       (fo::u32x4*)dst, (const fo::u32x4*)src, n_vec);
+    return check_hip(hipGetLastError(), "copy kernel launch");
+}
+
+}  // extern "C"

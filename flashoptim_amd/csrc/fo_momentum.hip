@@ -1,0 +1,154 @@
+// Fused SGD / SGDW / Nesterov / Lion step kernels (and the momentum-free SGD step) for gfx950 with their C
+// entry points (ref: /root/reference/flashoptim/optimizers.py:1447-1465, 1535-1719, cited as "ref:").
+#include "fo_step.h"
+
+namespace fo {
+
+// ------------------------------------------------------------------------------------------------
+// SGD / SGDW / Nesterov / Lion / momentum-free SGD (ref:1586-1719, 1447-1465)
+// ------------------------------------------------------------------------------------------------
+enum { KIND_SGD = 0, KIND_LION = 1, KIND_PLAIN = 2 };
+
+struct MomentumHyper {
+    float lr, mom_coef, update_coef, one_m_mom_coef, one_m_update_coef, wd, one_m_wd;
+    int decoupled, nesterov;
+    int apply_decay;  // momentum-free branch only: the reference skips both decays when weight_decay == 0
+};
+
+template <int DT, int ECCB, bool QUANT, int KIND, bool FAST>
+__device__ __forceinline__ void momentum_lane(const TensorPtrs& t, int64_t first, const MomentumHyper& h,
+                                              const float* lut_lane) {
+    constexpr int PB = DTypeInfo<DT>::bytes;
+    constexpr int SB = (KIND == KIND_PLAIN) ? 0 : (QUANT ? 1 : PB);
+    const int64_t n = t.n;
+
+    Pack<PB> praw, graw;
+    Pack<ECCB> eraw;
+    Pack<SB> mraw;
+    load_lane<PB, FAST>(graw, t.grad, first, n);
+    load_lane<PB, FAST>(praw, t.param, first, n);
+    load_lane<ECCB, FAST>(eraw, t.ecc, first, n);
+    load_lane<SB, FAST>(mraw, t.mom, first, n);
+    const bool live_group = FAST || first < n;
+    const int64_t group = first >> 5;
+    float sm = 1.0f;
+    if constexpr (QUANT && KIND != KIND_PLAIN) {
+        if (live_group) sm = f16_bits_to_f32(t.mom_scales[group]);               // ref:1645-1646
+    }
+
+    float p[kLaneElems], m[kLaneElems];
+    read_master<DT, ECCB>(p, praw, eraw);
+
+    float am = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kLaneElems; ++k) {
+        float g = widen<DT>(graw, k);
+        float pk = p[k];
+        if constexpr (KIND == KIND_PLAIN) {
+            if (h.apply_decay && !h.decoupled) g = g + pk * h.wd;                // ref:1452-1453
+            if (h.apply_decay && h.decoupled) pk = pk * h.one_m_wd;              // ref:1454-1455
+            pk = pk - g * h.lr;                                                  // ref:1456
+        } else {
+            if (KIND == KIND_SGD && !h.decoupled) g = g + pk * h.wd;             // ref:1639-1640
+            float mo;
+            if constexpr (QUANT) mo = lut_lane[byte_of(mraw, k) * 32] * sm;      // ref:1648-1657
+            else mo = widen<DT>(mraw, k);                                        // ref:1660-1661
+            float mn;
+            if constexpr (KIND == KIND_LION) {
+                const float u = (mo * h.update_coef) + (g * h.one_m_update_coef);     // ref:1667
+                const float sgn = (u > 0.0f) ? 1.0f : ((u < 0.0f) ? -1.0f : 0.0f);   // ref:1668
+                mn = (mo * h.mom_coef) + (g * h.one_m_mom_coef);                      // ref:1669
+                pk = pk * h.one_m_wd;                                                 // ref:1675
+                pk = pk - sgn * h.lr;                                                 // ref:1676
+            } else {
+                mn = mo * h.mom_coef + g * h.update_coef;                             // ref:1671
+                if (h.decoupled) pk = pk * h.one_m_wd;                                // ref:1678-1679
+                if (h.nesterov) pk = pk - (g + h.mom_coef * mn) * h.lr;               // ref:1680-1681
+                else pk = pk - mn * h.lr;                                             // ref:1682-1683
+            }
+            m[k] = mn;
+            am = fmaxf(am, fabsf(mn));
+        }
+        p[k] = pk;
+    }
+
+    Pack<ECCB> eout;
+    write_master<DT, ECCB>(p, praw, eout);                                       // ref:1684-1694
+    store_lane<PB, FAST>(praw, t.param, first, n);
+    store_lane<ECCB, FAST>(eout, t.ecc, first, n);
+
+    if constexpr (KIND != KIND_PLAIN) {
+        if constexpr (QUANT) {
+            am = fmaxf(fmaxf(am, pair_swap(am)), 1e-12f);                        // ref:1702-1703
+            quantize_mom(m, am, mraw);
+            store_lane<1, FAST>(mraw, t.mom, first, n);
+            if (live_group && (threadIdx.x & 1) == 0) t.mom_scales[group] = f32_to_f16_bits(am);  // ref:1713-1716
+        } else {
+            narrow_all<DT>(m, mraw);                                             // ref:1717-1719
+            store_lane<SB, FAST>(mraw, t.mom, first, n);
+        }
+    }
+}
+
+
+template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumOp {
+    using Hyper = MomentumHyper;
+    static constexpr bool kNeedsLut = QUANT && KIND != KIND_PLAIN;
+    template <bool FAST>
+    __device__ __forceinline__ static void lane(const TensorPtrs& t, int64_t first, const Hyper& h, const float* lut) {
+        momentum_lane<DT, ECCB, QUANT, KIND, FAST>(t, first, h, lut);
+    }
+};
+
+}  // namespace fo
+
+namespace {
+using namespace fo_host;
+
+template <int DT, int EB, bool Q> using SgdOp = fo::MomentumOp<DT, EB, Q, fo::KIND_SGD>;
+template <int DT, int EB, bool Q> using LionOp = fo::MomentumOp<DT, EB, Q, fo::KIND_LION>;
+template <int DT, int EB, bool Q> using PlainOp = fo::MomentumOp<DT, EB, Q, fo::KIND_PLAIN>;
+
+fo::MomentumHyper make_momentum_hyper(float lr, float mom_coef, float update_coef, float wd, int decoupled, int nesterov) {
+    fo::MomentumHyper h;
+    h.lr = lr; h.mom_coef = mom_coef; h.update_coef = update_coef;
+    h.one_m_mom_coef = 1.0f - mom_coef; h.one_m_update_coef = 1.0f - update_coef;
+    h.wd = wd; h.one_m_wd = 1.0f - wd;
+    h.decoupled = decoupled ? 1 : 0; h.nesterov = nesterov ? 1 : 0;
+    h.apply_decay = wd > 0.0f ? 1 : 0;
+    return h;
+}
+
+}  // namespace
+
+extern "C" {
+int fo_momentum_step(void* mom, void* mom_scales, void* param, const void* grad, void* ecc, int64_t n, int dtype,
+                     int ecc_bytes, int quantized, float lr, float mom_coef, float update_coef, float weight_decay,
+                     int decoupled, int nesterov, int do_lion, void* stream) {
+    if (int rc = validate_common(param, grad, ecc, n, dtype, ecc_bytes)) return rc;
+    if (n == 0) return 0;  // ref:1551-1553
+    if (int rc = validate_state(mom, mom_scales, quantized, dtype, "mom")) return rc;
+    fo::TensorPtrs t{param, grad, ecc_bytes ? ecc : nullptr, mom, (uint16_t*)mom_scales, nullptr, nullptr, n};
+    SingleLauncher<fo::MomentumHyper> L{t, make_momentum_hyper(lr, mom_coef, update_coef, weight_decay, decoupled, nesterov), (hipStream_t)stream};
+    return do_lion ? dispatch<LionOp>(dtype, ecc_bytes, quantized, L) : dispatch<SgdOp>(dtype, ecc_bytes, quantized, L);
+}
+
+int fo_sgd_plain_step(void* param, const void* grad, void* ecc, int64_t n, int dtype, int ecc_bytes, float lr,
+                      float weight_decay, int decoupled, void* stream) {
+    if (int rc = validate_common(param, grad, ecc, n, dtype, ecc_bytes)) return rc;
+    if (n == 0) return 0;
+    fo::TensorPtrs t{param, grad, ecc_bytes ? ecc : nullptr, nullptr, nullptr, nullptr, nullptr, n};
+    SingleLauncher<fo::MomentumHyper> L{t, make_momentum_hyper(lr, 0.0f, 1.0f, weight_decay, decoupled, 0), (hipStream_t)stream};
+    return dispatch<PlainOp>(dtype, ecc_bytes, 0, L);
+}
+
+int fo_multi_momentum_step(const fo_tensor_desc* descs, int64_t n_tensors, const fo_chunk* chunks, int64_t n_chunks,
+                           int dtype, int ecc_bytes, int quantized, float lr, float mom_coef, float update_coef,
+                           float weight_decay, int decoupled, int nesterov, int do_lion, void* stream) {
+    if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
+    if (n_chunks == 0) return 0;
+    MultiLauncher<fo::MomentumHyper> L{descs, chunks, n_chunks, make_momentum_hyper(lr, mom_coef, update_coef, weight_decay, decoupled, nesterov), (hipStream_t)stream};
+    return do_lion ? dispatch<LionOp>(dtype, ecc_bytes, quantized, L) : dispatch<SgdOp>(dtype, ecc_bytes, quantized, L);
+}
+
+}  // extern "C"

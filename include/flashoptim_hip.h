@@ -1,0 +1,152 @@
+/*
+ * flashoptim_hip.h -- C ABI of libflashoptim_hip.so, the gfx950 (MI355X) implementation of FlashOptim's
+ * fused optimizer-step hot path.
+ *
+ * Every entry point takes raw device pointers, sizes, fp32 scalars and a HIP stream (as void*); none takes
+ * a torch type, allocates tensor memory or synchronises with the host.  All work is enqueued on `stream`
+ * and mutates the caller's buffers in place, exactly as the reference's Triton launch wrappers do.
+ * Return value: 0 on success, otherwise a negative FO_ERR_* code or a positive hipError_t; the text of the
+ * last failure on the calling thread is available from fo_last_error().  Nothing throws across the ABI.
+ *
+ * "ref:" cites /root/reference/flashoptim/optimizers.py, the interface each symbol replaces.
+ *
+ * Layout contract shared by all entry points (ref:2476-2484, 1625-1646):
+ *   - tensors are flat and contiguous; element i of the parameter pairs with element i of grad, ecc, codes;
+ *   - a quantisation group is 32 consecutive elements counted from element 0 of the tensor; scales are
+ *     fp16, one per group, ceil(n/32) entries; a short last group is scaled by its own absmax;
+ *   - first-moment codes are int8 (softsign companding), second-moment codes uint8 (of sqrt(v));
+ *   - ECC is int8 (24-bit master) or int16 (32-bit master), absent for fp32 parameters.
+ */
+#ifndef FLASHOPTIM_HIP_H
+#define FLASHOPTIM_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* parameter / gradient element type (ref:60-64 _TORCH_DTYPE_TO_TRITON_DTYPE) */
+enum fo_dtype { FO_F32 = 0, FO_BF16 = 1, FO_F16 = 2 };
+
+enum fo_error {
+    FO_OK = 0,
+    FO_ERR_INVALID_ARGUMENT = -1, /* bad enum, null pointer, negative size, misaligned scale pointer ... */
+    FO_ERR_UNSUPPORTED = -2,      /* e.g. ECC requested for an fp32 parameter */
+    FO_ERR_NO_DEVICE = -3
+};
+
+/* Library / device identification. */
+int fo_version(void);                    /* 100*major + minor */
+const char *fo_last_error(void);         /* thread-local, never NULL */
+int fo_device_compute_units(int device); /* multiprocessor count, <0 on error (ref:2976-2980 _get_sm_count) */
+
+/*
+ * Fused Adam / AdamW step on one tensor.  Replaces _fused_adam_step + _triton_adam_kernel
+ * (ref:2203-2251, 2255-2438).
+ *   mom, var        : quantized != 0 -> int8 / uint8 codes; else tensors of the parameter dtype
+ *   mom_scales,
+ *   var_scales      : fp16[ceil(n/32)] when quantized, ignored otherwise (may be NULL)
+ *   param, grad     : `dtype` elements; grad is read only
+ *   ecc             : int8 (ecc_bytes 1) / int16 (ecc_bytes 2) / NULL (ecc_bytes 0)
+ *   weight_decay    : what the reference launcher passes: already multiplied by lr (or lr/initial_lr) for the
+ *                     decoupled optimizers, the raw L2 coefficient otherwise (ref:1894-1898)
+ *   step            : 1-based step count used for bias correction (ref:2368-2369)
+ */
+int fo_adam_step(void *mom, void *mom_scales, void *var, void *var_scales, void *param, const void *grad,
+                 void *ecc, int64_t n, int dtype, int ecc_bytes, int quantized, float lr, float beta1,
+                 float beta2, float eps, float weight_decay, int decoupled, int step, void *stream);
+
+/*
+ * Fused SGD / SGDW / Nesterov / Lion step on one tensor.  Replaces _fused_momentum_step +
+ * _triton_momentum_kernel (ref:1535-1579, 1586-1719).  Lion: mom_coef = beta2, update_coef = beta1,
+ * do_lion = 1 (ref:1313-1317); SGD: mom_coef = momentum, update_coef = 1 - dampening (ref:1432-1433).
+ */
+int fo_momentum_step(void *mom, void *mom_scales, void *param, const void *grad, void *ecc, int64_t n,
+                     int dtype, int ecc_bytes, int quantized, float lr, float mom_coef, float update_coef,
+                     float weight_decay, int decoupled, int nesterov, int do_lion, void *stream);
+
+/*
+ * Momentum-free SGD step (no state tensor).  Replaces the eager branch the reference takes when
+ * momentum == 0 (ref:1447-1465): both decays are skipped when weight_decay == 0.
+ */
+int fo_sgd_plain_step(void *param, const void *grad, void *ecc, int64_t n, int dtype, int ecc_bytes, float lr,
+                      float weight_decay, int decoupled, void *stream);
+
+/*
+ * Multi-tensor launch: one grid over many tensors of ragged sizes (no counterpart in the reference, which
+ * launches once per tensor from FlashOptimizer.step, ref:770-785; results are bit-identical to calling the
+ * single-tensor entry point on every tensor).
+ *
+ * `descs` is a DEVICE array of n_tensors descriptors; `chunks` is a DEVICE array of n_chunks work items
+ * produced by fo_build_chunks (host) and copied by the caller.  All tensors of one call share dtype,
+ * ecc_bytes, quantized and the scalar hyper-parameters (callers bucket by those).
+ */
+typedef struct fo_tensor_desc {
+    void *param;
+    const void *grad;
+    void *ecc;        /* NULL when ecc_bytes == 0 */
+    void *mom;        /* NULL for fo_multi_sgd_plain_step */
+    void *mom_scales; /* NULL when not quantized */
+    void *var;        /* Adam only */
+    void *var_scales; /* Adam only, NULL when not quantized */
+    int64_t n;        /* elements in this tensor */
+} fo_tensor_desc;
+
+typedef struct fo_chunk {
+    int32_t tensor;     /* index into descs */
+    int32_t first_tile; /* first 4096-element tile of the tensor covered by this chunk */
+    int32_t n_tiles;    /* tiles covered (>= 1) */
+    int32_t reserved;
+} fo_chunk;
+
+#define FO_TILE_ELEMS 4096
+
+/* Host helper: number of chunks fo_build_chunks will emit for these tensor lengths (0-length tensors emit
+ * none).  tiles_per_chunk <= 0 selects the library default. */
+int64_t fo_count_chunks(const int64_t *numels, int64_t n_tensors, int tiles_per_chunk);
+/* Host helper: fills `out` (host memory, capacity >= fo_count_chunks) and returns the count, <0 on error. */
+int64_t fo_build_chunks(const int64_t *numels, int64_t n_tensors, int tiles_per_chunk, fo_chunk *out,
+                        int64_t capacity);
+
+int fo_multi_adam_step(const fo_tensor_desc *descs, int64_t n_tensors, const fo_chunk *chunks, int64_t n_chunks,
+                       int dtype, int ecc_bytes, int quantized, float lr, float beta1, float beta2, float eps,
+                       float weight_decay, int decoupled, int step, void *stream);
+
+int fo_multi_momentum_step(const fo_tensor_desc *descs, int64_t n_tensors, const fo_chunk *chunks,
+                           int64_t n_chunks, int dtype, int ecc_bytes, int quantized, float lr, float mom_coef,
+                           float update_coef, float weight_decay, int decoupled, int nesterov, int do_lion,
+                           void *stream);
+
+/*
+ * Standalone group codec.  Replaces quantize / dequantize and their kernels (ref:2446-2538, 2541-2676).
+ *   x            : `x_dtype` elements
+ *   codes        : int8 when is_signed, uint8 otherwise
+ *   scales       : fp16[ceil(n/32)]
+ */
+int fo_quantize(const void *x, int x_dtype, void *codes, void *scales, int64_t n, int is_signed, int do_sqrt,
+                int softsign, void *stream);
+int fo_dequantize(const void *codes, const void *scales, float *out, int64_t n, int is_signed, int do_sqrt,
+                  int softsign, void *stream);
+
+/*
+ * Standalone ECC.  fo_ecc_join replaces reconstruct_fp32_param (ref:2835-2892, kernel 2779-2803);
+ * fo_ecc_split replaces compute_ecc_bits (ref:2895-2970, kernel 2806-2832).  narrow_dtype is FO_BF16 or
+ * FO_F16; ecc_bytes is 1 or 2.
+ */
+int fo_ecc_join(const void *narrow, int narrow_dtype, const void *ecc, int ecc_bytes, float *out, int64_t n,
+                void *stream);
+int fo_ecc_split(const float *x, const void *narrow, int narrow_dtype, void *ecc, int ecc_bytes, int64_t n,
+                 void *stream);
+
+/*
+ * Measurement aid: a plain device-to-device copy kernel (128-bit loads and stores, same launch geometry as
+ * the step kernels) used to calibrate hardware byte counters and to show the attainable HBM rate next to the
+ * step kernels.  n_bytes must be a multiple of 16 and both pointers 16-byte aligned.
+ */
+int fo_copy_bytes(void *dst, const void *src, int64_t n_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHOPTIM_HIP_H */

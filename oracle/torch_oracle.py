@@ -253,7 +253,7 @@ def _store_state(
 def _read_master(param: torch.Tensor, ecc: Optional[torch.Tensor]) -> torch.Tensor:
     if ecc is not None:
         return ecc_join_ref(param, ecc)  # ref:2300-2307
-    return param.to(torch.float32)  # ref:2308-2309
+    return param.to(torch.float32, copy=True)  # ref:2308-2309 (a copy, so the caller keeps the value from before the step)
 
 
 def _write_master(param: torch.Tensor, ecc: Optional[torch.Tensor], p: torch.Tensor) -> None:
@@ -276,11 +276,14 @@ def adam_step_ref(
     weight_decay: float,
     decoupled: bool,
     step: int,
-) -> None:
+) -> dict:
     """``_triton_adam_kernel`` (ref:2255-2438) on flat, contiguous CPU tensors, in place.
 
     ``weight_decay`` is what the launcher passes: already multiplied by lr (or lr/initial_lr) in
     double for the decoupled optimizers (ref:1894-1898).
+
+    Returns the fp32 intermediates a parity test needs to tell a genuine difference from a rounding
+    coin-flip: the master before and after the update and the moments before requantisation.
     """
     lr, b1, b2, eps, wd = f32(lr), f32(beta1), f32(beta2), f32(eps), f32(weight_decay)
     one_m_b1 = f32(np.float32(1.0) - np.float32(b1))
@@ -291,6 +294,7 @@ def adam_step_ref(
 
     g = grad.reshape(-1).to(torch.float32)  # ref:2297-2298
     p = _read_master(param.reshape(-1), None if ecc is None else ecc.reshape(-1))
+    p_before = p
     if not decoupled:
         g = g + p * wd  # ref:2310-2311
     m = _load_state(mom, signed=True, sqrt=False, softsign=True)  # ref:2325-2343
@@ -306,6 +310,7 @@ def adam_step_ref(
     _write_master(param.reshape(-1), None if ecc is None else ecc.reshape(-1), p)
     _store_state(mom, m, signed=True, sqrt=False, softsign=True)  # ref:2390-2434
     _store_state(var, v, signed=False, sqrt=True, softsign=False)
+    return {"p_before": p_before, "p_after": p, "m": m, "v": v}
 
 
 def momentum_step_ref(
@@ -320,7 +325,7 @@ def momentum_step_ref(
     decoupled: bool = False,
     nesterov: bool = False,
     do_lion: bool = False,
-) -> None:
+) -> dict:
     """``_triton_momentum_kernel`` (ref:1586-1719), in place.
 
     Lion: ``mom_coef = beta2``, ``update_coef = beta1`` (ref:1313-1317).  SGD: ``mom_coef =
@@ -334,6 +339,7 @@ def momentum_step_ref(
 
     g = grad.reshape(-1).to(torch.float32)  # ref:1626-1627
     p = _read_master(param.reshape(-1), eccf)  # ref:1628-1638
+    p_before = p
 
     if mom is None:
         # ref:1452-1456: the eager branch skips both decays when weight_decay == 0.
@@ -343,7 +349,7 @@ def momentum_step_ref(
             p = p * one_m_wd
         p = p - g * lr
         _write_master(param.reshape(-1), eccf, p)
-        return
+        return {"p_before": p_before, "p_after": p}
 
     if not do_lion and not decoupled:
         g = g + p * wd  # ref:1639-1640
@@ -366,3 +372,4 @@ def momentum_step_ref(
             p = p - m * lr  # ref:1682-1683
     _write_master(param.reshape(-1), eccf, p)  # ref:1684-1694
     _store_state(mom, m, signed=True, sqrt=False, softsign=True)  # ref:1697-1719
+    return {"p_before": p_before, "p_after": p, "m": m}

@@ -1,0 +1,272 @@
+"""GPU parity of the HIP kernels (through the C ABI, via flashoptim_amd.kernels) against the CPU oracle."""
+
+import pytest
+import torch
+
+from oracle import c_oracle as C
+from oracle import torch_oracle as T
+from tests import parity
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+MODES = [(True, False, False), (True, False, True), (False, False, False), (False, True, False)]
+SIZES = [1, 5, 31, 32, 33, 1000, 4095, 4096, 4097, 3 * 4096 + 555, 1 << 18]
+
+
+def _k():
+    from flashoptim_amd import kernels
+    return kernels
+
+
+def _rand(n, scale, seed):
+    return torch.randn(n, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+# ------------------------------------------------------------------------------------ standalone codec
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("signed,sqrt,softsign", MODES)
+def test_quantize_dequantize_bit_exact(dtype, signed, sqrt, softsign):
+    k = _k()
+    for i, n in enumerate(SIZES):
+        x = (_rand(n, 3.0, i) * (0.01 if i % 3 == 0 else 1.0)).to(dtype)
+        if not signed:
+            x = x.abs()
+        codes, scales = k.quantize(x.to(DEV), signed=signed, sqrt=sqrt, softsign=softsign)
+        rc, rs = C.quantize(x, signed, sqrt, softsign)
+        assert codes.shape == x.shape and scales.numel() == (n + 31) // 32
+        assert torch.equal(codes.cpu(), rc), (n, "codes")
+        assert parity.bits_equal(scales, rs), (n, "scales")
+        back = k.dequantize(codes, scales, signed=signed, sqrt=sqrt, softsign=softsign)
+        assert parity.bits_equal(back, C.dequantize(rc, rs, signed, sqrt, softsign)), (n, "dequantize")
+
+
+def test_quantize_unaligned_view_and_2d():
+    k = _k()
+    base = _rand(10001, 1.0, 3).to(torch.bfloat16).to(DEV)
+    view = base[1:]  # 2-byte offset: not 16-byte aligned -> guarded path
+    codes, scales = k.quantize(view)
+    rc, rs = C.quantize(base.cpu()[1:].contiguous())
+    assert torch.equal(codes.cpu(), rc) and parity.bits_equal(scales, rs)
+    x2 = _rand(64 * 33, 1.0, 4).view(64, 33).to(DEV)
+    c2, s2 = k.quantize(x2)
+    assert c2.shape == (64, 33)
+    rc2, rs2 = C.quantize(x2.cpu())
+    assert torch.equal(c2.cpu(), rc2) and parity.bits_equal(s2, rs2)
+
+
+def test_dequantize_every_code_bit_exact():
+    """All 256 code bytes x several scales, signed+softsign and unsigned+sqrt: the table behind the fused
+    kernels' dequantisation must equal IEEE evaluation of the reference formula."""
+    k = _k()
+    for signed, sqrt, softsign in MODES:
+        codes = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+        codes = codes.view(torch.int8) if signed else codes
+        scales = torch.tensor([1.0, 0.37, 6.1e-5, 3.2e-5, 5.96e-8, 1234.0, 0.0, 65504.0], dtype=torch.float16)
+        got = k.dequantize(codes.to(DEV), scales.to(DEV), signed=signed, sqrt=sqrt, softsign=softsign)
+        assert parity.bits_equal(got, C.dequantize(codes, scales, signed, sqrt, softsign))
+
+
+# ------------------------------------------------------------------------------------- standalone ECC
+
+
+@pytest.mark.parametrize("narrow", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("ecc_dtype,width", [(torch.int8, 3), (torch.int16, 4)])
+def test_ecc_split_join_bit_exact(narrow, ecc_dtype, width):
+    k = _k()
+    g = torch.Generator().manual_seed(7)
+    for n in [1, 17, 4096, 4097, 1 << 18]:
+        mags = torch.exp(torch.empty(n).uniform_(-30, 10, generator=g))
+        x = mags * torch.where(torch.rand(n, generator=g) < 0.5, -1.0, 1.0)
+        x[: min(n, 6)] = torch.tensor([0.0, 1.0, 1 + 2.0**-8, -(1 + 2.0**-9), 2.0**-130, 1e-40])[: min(n, 6)]
+        if narrow == torch.float16:
+            x = x.clamp(-60000, 60000)
+        nar = x.to(narrow)
+        ecc = k.compute_ecc_bits(x.to(DEV), nar.to(DEV), master_bytewidth=width)
+        ref = C.ecc_split(x, nar, ecc_dtype)
+        assert ecc.dtype == ecc_dtype and torch.equal(ecc.cpu(), ref), n
+        rec = k.reconstruct_fp32_param(nar.to(DEV), ecc)
+        assert parity.bits_equal(rec, C.ecc_join(nar, ref)), n
+
+
+def test_ecc_join_every_int16_value():
+    k = _k()
+    ecc = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16)
+    for val in [1.0, -3.5, 2.0**-126, 0.0, 1e-3]:
+        nar = torch.full((65536,), val).to(torch.bfloat16)
+        assert parity.bits_equal(k.reconstruct_fp32_param(nar.to(DEV), ecc.to(DEV)), C.ecc_join(nar, ecc))
+
+
+def test_wrapper_errors():
+    k = _k()
+    with pytest.raises(ValueError):
+        k.reconstruct_fp32_param(torch.zeros(4, device=DEV), torch.zeros(4, dtype=torch.int8, device=DEV))
+    with pytest.raises(ValueError):
+        k.reconstruct_fp32_param(torch.zeros(4, device=DEV, dtype=torch.bfloat16), torch.zeros(4, dtype=torch.int32, device=DEV))
+    with pytest.raises(ValueError):
+        k.compute_ecc_bits(torch.zeros(4, device=DEV, dtype=torch.bfloat16), torch.zeros(4, device=DEV, dtype=torch.bfloat16))
+    with pytest.raises(ValueError):
+        k.compute_ecc_bits(torch.zeros(4, device=DEV), torch.zeros(4, device=DEV, dtype=torch.bfloat16), master_bytewidth=2)
+    with pytest.raises(NotImplementedError):
+        k.quantize(torch.zeros(4))
+
+
+# ---------------------------------------------------------------------------------------- fused steps
+
+VARIANTS = [
+    (torch.bfloat16, torch.int8), (torch.bfloat16, torch.int16), (torch.bfloat16, None),
+    (torch.float16, torch.int8), (torch.float16, torch.int16), (torch.float16, None), (torch.float32, None),
+]
+
+
+class _Case:
+    """State of one tensor on the CPU (oracle side) mirrored on the GPU."""
+
+    def __init__(self, n, dtype, ecc_dtype, quantized, n_states, seed, offset=0):
+        self.n, self.dtype, self.quantized = n, dtype, quantized
+        self.p = _rand(n, 0.02, seed).to(dtype)
+        self.ecc = None if ecc_dtype is None else torch.zeros(n, dtype=ecc_dtype)
+        self.states = [T.MomentState.zeros(n, i == 0, quantized, dtype) for i in range(n_states)]
+        self.offset = offset
+        self.gp = self._dev(self.p)
+        self.gecc = None if self.ecc is None else self._dev(self.ecc)
+        self.gstates = [
+            (self._dev(s.codes), s.scales.to(DEV)) if quantized else (self._dev(s.plain), None) for s in self.states
+        ]
+
+    def _dev(self, t):
+        # offset > 0 places the tensor at a misaligned address inside a larger buffer (guarded path)
+        if self.offset == 0:
+            return t.to(DEV)
+        buf = torch.zeros(t.numel() + self.offset, dtype=t.dtype, device=DEV)
+        buf[self.offset:].copy_(t)
+        return buf[self.offset:]
+
+    def resync_oracle(self):
+        """Copy the GPU state to the CPU so the next comparison starts from identical inputs."""
+        self.p.copy_(self.gp.cpu())
+        if self.ecc is not None:
+            self.ecc.copy_(self.gecc.cpu())
+        for s, (a, b) in zip(self.states, self.gstates):
+            if self.quantized:
+                s.codes.copy_(a.cpu())
+                s.scales.copy_(b.cpu())
+            else:
+                s.plain.copy_(a.cpu())
+
+    def compare(self, what, info):
+        """`info`: the oracle's intermediates of the step just taken."""
+        parity.check_master(self.gp, self.gecc, self.p, self.ecc, what,
+                            step_size=(info["p_after"] - info["p_before"]).abs())
+        stats = []
+        for i, (s, (a, b)) in enumerate(zip(self.states, self.gstates)):
+            if self.quantized:
+                band = parity.near_tie_mom(info["m"]) if i == 0 else parity.near_tie_var(info["v"])
+                stats.append(parity.check_codes(a, s.codes, f"{what} state{i}", near_tie=band))
+                parity.check_scales(b, s.scales, f"{what} state{i}")
+            else:
+                d = (a.cpu().double() - s.plain.double()).abs()
+                assert bool((d <= parity.ulp_of(s.plain) * 1.0000001).all()), f"{what} state{i}: more than one ulp"
+        return stats
+
+
+def _adam_steps(n, dtype, ecc_dtype, quantized, decoupled, steps, seed, offset=0, grad_scale=1e-3):
+    k = _k()
+    c = _Case(n, dtype, ecc_dtype, quantized, 2, seed, offset)
+    lr, b1, b2, eps = 1e-3, 0.9, 0.999, 1e-8
+    wd = 0.01 * lr if decoupled else 0.01
+    worst_raw = worst_filtered = 0.0
+    for step in range(1, steps + 1):
+        g = _rand(n, grad_scale, 1000 * seed + step).to(dtype)
+        gg = c._dev(g)
+        (m, ms), (v, vs) = c.gstates
+        k._fused_adam_step(m, ms, v, vs, c.gp, gg, c.gecc, lr, b1, b2, eps, wd, decoupled, step, quantize_optim_states=quantized)
+        info = T.adam_step_ref(c.states[0], c.states[1], c.p, g, c.ecc, lr, b1, b2, eps, wd, decoupled, step)
+        stats = c.compare(f"adam n={n} {dtype} ecc={ecc_dtype} q={quantized} step={step}", info)
+        for raw, filt in stats:
+            worst_raw, worst_filtered = max(worst_raw, raw), max(worst_filtered, filt)
+        c.resync_oracle()
+    return worst_raw, worst_filtered
+
+
+@pytest.mark.parametrize("dtype,ecc_dtype", VARIANTS)
+@pytest.mark.parametrize("quantized", [True, False])
+@pytest.mark.parametrize("decoupled", [True, False])
+def test_adam_step_matches_oracle(dtype, ecc_dtype, quantized, decoupled):
+    for i, n in enumerate([1, 31, 33, 1000, 4096, 4097 + 4096, (1 << 16) + 17]):
+        _adam_steps(n, dtype, ecc_dtype, quantized, decoupled, steps=4, seed=i + 1)
+
+
+def test_adam_headline_config_code_mismatch_rate():
+    """bf16 + int8 ECC + quantised AdamW on 2^20 and 2^20+17 elements, 10 steps: the sizes used for the
+    parity sub-check of the 2^30 throughput run."""
+    for n in [1 << 20, (1 << 20) + 17]:
+        raw, filtered = _adam_steps(n, torch.bfloat16, torch.int8, True, True, steps=10, seed=5)
+        print(f"n={n}: worst per-step code mismatch fraction raw {raw:.3e}, outside the tie band {filtered:.3e}")
+        assert filtered < parity.CODE_MISMATCH_FRACTION
+
+
+def test_adam_unaligned_pointers():
+    _adam_steps(5000, torch.bfloat16, torch.int8, True, True, steps=3, seed=9, offset=3)
+    _adam_steps(5000, torch.float32, None, True, True, steps=3, seed=9, offset=1)
+
+
+def test_adam_large_and_tiny_gradients():
+    # 1e-3-sized gradients put sqrt(v) scales into the fp16 subnormal range; 10-sized ones far above it
+    _adam_steps(1 << 14, torch.bfloat16, torch.int16, True, True, steps=5, seed=11, grad_scale=10.0)
+    _adam_steps(1 << 14, torch.bfloat16, torch.int8, True, True, steps=5, seed=12, grad_scale=1e-7)
+
+
+MOM_MODES = {
+    "lion": dict(lr=1e-4, mom_coef=0.99, update_coef=0.9, weight_decay=0.1 * 1e-4, do_lion=True),
+    "sgd": dict(lr=1e-2, mom_coef=0.9, update_coef=0.9, weight_decay=1e-4),
+    "sgd_nesterov": dict(lr=1e-2, mom_coef=0.9, update_coef=1.0, weight_decay=1e-4, nesterov=True),
+    "sgdw": dict(lr=1e-2, mom_coef=0.9, update_coef=1.0, weight_decay=1e-4 * 1e-2, decoupled=True),
+    "sgdw_nesterov": dict(lr=1e-2, mom_coef=0.9, update_coef=1.0, weight_decay=1e-4 * 1e-2, decoupled=True, nesterov=True),
+}
+
+
+@pytest.mark.parametrize("dtype,ecc_dtype", VARIANTS)
+@pytest.mark.parametrize("quantized", [True, False])
+@pytest.mark.parametrize("mode", list(MOM_MODES))
+def test_momentum_step_matches_oracle(dtype, ecc_dtype, quantized, mode):
+    k = _k()
+    kw = MOM_MODES[mode]
+    for i, n in enumerate([1, 33, 1000, 4097, (1 << 16) + 17]):
+        c = _Case(n, dtype, ecc_dtype, quantized, 1, seed=20 + i)
+        for step in range(1, 5):
+            g = _rand(n, 1e-3, 77 * i + step).to(dtype)
+            (m, ms), = c.gstates
+            k._fused_momentum_step(m, ms, c.gp, g.to(DEV), c.gecc, quantize_optim_states=quantized, **kw)
+            info = T.momentum_step_ref(c.states[0], c.p, g, c.ecc, **kw)
+            c.compare(f"{mode} n={n} {dtype} ecc={ecc_dtype} q={quantized} step={step}", info)
+            c.resync_oracle()
+
+
+@pytest.mark.parametrize("dtype,ecc_dtype", VARIANTS)
+@pytest.mark.parametrize("decoupled,wd", [(False, 0.0), (False, 1e-2), (True, 1e-4)])
+def test_plain_sgd_matches_oracle(dtype, ecc_dtype, decoupled, wd):
+    k = _k()
+    for i, n in enumerate([1, 33, 4097, (1 << 16) + 17]):
+        c = _Case(n, dtype, ecc_dtype, False, 0, seed=40 + i)
+        for step in range(1, 4):
+            g = _rand(n, 1e-2, 99 * i + step).to(dtype)
+            k._sgd_plain_step(c.gp, g.to(DEV), c.gecc, 1e-2, wd, decoupled)
+            info = T.momentum_step_ref(None, c.p, g, c.ecc, 1e-2, 0.0, 1.0, wd, decoupled=decoupled)
+            c.compare(f"plain sgd n={n} step={step}", info)
+            c.resync_oracle()
+
+
+def test_zero_gradients_change_nothing():
+    k = _k()
+    n = 10000
+    c = _Case(n, torch.bfloat16, torch.int8, True, 2, seed=60)
+    p0 = c.gp.clone()
+    (m, ms), (v, vs) = c.gstates
+    for step in range(1, 4):
+        k._fused_adam_step(m, ms, v, vs, c.gp, torch.zeros(n, dtype=torch.bfloat16, device=DEV), c.gecc, 1e-3, 0.9, 0.999,
+                           1e-8, 0.0, True, step)
+    assert torch.equal(c.gp, p0) and m.eq(0).all() and v.eq(0).all() and c.gecc.eq(0).all()
+    assert ms.eq(0).all() and vs.eq(0).all()
