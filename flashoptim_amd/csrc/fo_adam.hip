@@ -3,34 +3,37 @@
 #include "fo_step.h"
 
 #include <cmath>
+#include <limits>
 
 namespace fo {
 
-// ------------------------------------------------------------------------------------------------
-// Adam / AdamW (ref:2255-2438)
-// ------------------------------------------------------------------------------------------------
+// Per-launch constants.  Scalars arrive as fp32 like the reference's kernel arguments; 1 - x is formed in fp32
+// (ref:2357-2364).  The per-step bias corrections and the learning rate are folded on the host (in double,
+// rounded once) into the two constants of the update's denominator:
+//     lr * (m / bc1) / (sqrt(v / bc2) + eps)  ==  m / (sqrt(v) * den_scale + den_bias)
+//     den_scale = bc1 / (lr * sqrt(bc2)),  den_bias = eps * bc1 / lr
 struct AdamHyper {
-    float b1, one_m_b1, b2, one_m_b2, wd, one_m_wd;
-    float lr_over_bc1;   // lr / (1 - b1^step)
-    float rsqrt_bc2;     // 1 / sqrt(1 - b2^step)
-    float eps;
+    float b1, one_m_b1, one_m_b2, wd, one_m_wd;
+    float sqrt_b2_over_255;  // dequantised sqrt(v_old * b2) = code * scale * sqrt(b2) / 255
+    float b2;                // unquantised states only
+    float den_scale, den_bias;
 };
 
 template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool FAST>
-__device__ __forceinline__ void adam_lane(const TensorPtrs& t, int64_t first, const AdamHyper& h,
-                                          const float* lut_lane) {
+__device__ __forceinline__ void adam_lane(const TensorPtrs& t, int64_t first, const AdamHyper& h, const float* lut_lane) {
+    constexpr int EPL = DTypeInfo<DT>::epl;
     constexpr int PB = DTypeInfo<DT>::bytes;
     constexpr int SB = QUANT ? 1 : PB;  // state bytes per element
     const int64_t n = t.n;
 
-    Pack<PB> praw, graw;
-    Pack<ECCB> eraw;
-    Pack<SB> mraw, vraw;
-    load_lane<PB, FAST>(graw, t.grad, first, n);
-    load_lane<PB, FAST>(praw, t.param, first, n);
-    load_lane<ECCB, FAST>(eraw, t.ecc, first, n);
-    load_lane<SB, FAST>(mraw, t.mom, first, n);
-    load_lane<SB, FAST>(vraw, t.var, first, n);
+    Pack<PB, EPL> praw, graw;
+    Pack<ECCB, EPL> eraw;
+    Pack<SB, EPL> mraw, vraw;
+    load_lane<PB, EPL, FAST>(graw, t.grad, first, n);
+    load_lane<PB, EPL, FAST>(praw, t.param, first, n);
+    load_lane<ECCB, EPL, FAST>(eraw, t.ecc, first, n);
+    load_lane<SB, EPL, FAST>(mraw, t.mom, first, n);
+    load_lane<SB, EPL, FAST>(vraw, t.var, first, n);
     const bool live_group = FAST || first < n;  // the lane owns at least one real element
     const int64_t group = first >> 5;
     float sm = 1.0f, sv = 1.0f;  // masked scales read 1.0 (ref:2318-2323)
@@ -40,68 +43,71 @@ __device__ __forceinline__ void adam_lane(const TensorPtrs& t, int64_t first, co
             sv = f16_bits_to_f32(t.var_scales[group]);
         }
     }
+    // the EMA decay is folded into the group scale: one multiply per lane instead of one per element
+    const float sm_b1 = sm * h.b1;
+    const float sv_b2 = sv * h.sqrt_b2_over_255;
 
-    float p[kLaneElems], m[kLaneElems], r[kLaneElems], v[kLaneElems];
-    read_master<DT, ECCB>(p, praw, eraw);
+    float p[EPL], m[EPL], r[EPL], v[EPL];
+    read_master<DT, ECCB, EPL>(p, praw, eraw);
 
     float am = 0.0f, vm = 0.0f;
 #pragma unroll
-    for (int k = 0; k < kLaneElems; ++k) {
-        float g = widen<DT>(graw, k);
-        if constexpr (!DECOUPLED) g = g + p[k] * h.wd;                                   // ref:2310-2311
-        float mo, vo;
+    for (int k = 0; k < EPL; ++k) {
+        float g = widen<DT, EPL>(graw, k);
+        if constexpr (!DECOUPLED) g = g + p[k] * h.wd;                              // ref:2310-2311
+        float mn, vn;
         if constexpr (QUANT) {
-            mo = lut_lane[byte_of(mraw, k) * 32] * sm;                           // ref:2332-2343
-            const float s = code255_to_unit((float)byte_of(vraw, k)) * sv;       // ref:2333-2346
-            vo = s * s;                                                          // ref:2348
+            // m = dequant(m) * b1 + g * (1 - b1)   (ref:2332-2343, 2357)
+            mn = fmaf(StepLut::lookup(lut_lane, byte_of<EPL>(mraw, k)), sm_b1, g * h.one_m_b1);
+            // v = dequant(v) * b2 + g^2 * (1 - b2), dequant(v) = (code/255 * scale)^2   (ref:2333-2348, 2360)
+            const float s = (float)byte_of<EPL>(vraw, k) * sv_b2;
+            vn = fmaf(s, s, (g * g) * h.one_m_b2);
         } else {
-            mo = widen<DT>(mraw, k);                                             // ref:2351-2354
-            vo = widen<DT>(vraw, k);
+            // unquantised states: operation by operation as written in the reference, no contraction
+            mn = widen<DT, EPL>(mraw, k) * h.b1 + g * h.one_m_b1;                   // ref:2351-2357
+            vn = widen<DT, EPL>(vraw, k) * h.b2 + (g * g) * h.one_m_b2;             // ref:2360
         }
-        const float mn = mo * h.b1 + g * h.one_m_b1;                             // ref:2357
-        const float vn = vo * h.b2 + (g * g) * h.one_m_b2;                       // ref:2360
         float pk = p[k];
-        if constexpr (DECOUPLED) pk = pk * h.one_m_wd;                                   // ref:2363-2364
-        // p -= lr * (m/bc1) / (sqrt(v/bc2) + eps)  (ref:2368-2375), with sqrt(v) shared with the requantiser
+        if constexpr (DECOUPLED) pk = pk * h.one_m_wd;                              // ref:2363-2364
+        // p -= lr * (m/bc1) / (sqrt(v/bc2) + eps)  (ref:2368-2375); sqrt(v) is shared with the requantiser
         const float rk = __builtin_amdgcn_sqrtf(vn);
-        const float den = fmaf(rk, h.rsqrt_bc2, h.eps);
-        pk = fmaf(-(h.lr_over_bc1 * mn), __builtin_amdgcn_rcpf(den), pk);
+        const float den = fmaf(rk, h.den_scale, h.den_bias);
+        pk = fmaf(-mn, __builtin_amdgcn_rcpf(den), pk);
         p[k] = pk; m[k] = mn; r[k] = rk; v[k] = vn;
         am = fmaxf(am, fabsf(mn));
         vm = fmaxf(vm, vn);
     }
 
-    Pack<ECCB> eout;
-    write_master<DT, ECCB>(p, praw, eout);
-    store_lane<PB, FAST>(praw, t.param, first, n);
-    store_lane<ECCB, FAST>(eout, t.ecc, first, n);
+    Pack<ECCB, EPL> eout;
+    write_master<DT, ECCB, EPL>(p, praw, eout);
+    store_lane<PB, EPL, FAST>(praw, t.param, first, n);
+    store_lane<ECCB, EPL, FAST>(eout, t.ecc, first, n);
 
     if constexpr (QUANT) {
-        // group absmax over the lane pair (ref:2399-2404); sqrt is monotone, so the absmax of sqrt(v) is the
-        // correctly rounded root of max(v)
-        am = fmaxf(fmaxf(am, pair_swap(am)), 1e-12f);
-        vm = fmaxf(vm, pair_swap(vm));
-        const float av = fmaxf(sqrt_rn(vm), 1e-12f);
-        quantize_mom(m, am, mraw);
-        quantize_var(r, av, vraw);
-        store_lane<1, FAST>(mraw, t.mom, first, n);
-        store_lane<1, FAST>(vraw, t.var, first, n);
-        if (live_group && (threadIdx.x & 1) == 0) {                              // ref:2424-2434
+        // group absmax (ref:2399-2404); sqrt is monotone, so the absmax of sqrt(v) is the correctly rounded
+        // root of max(v)
+        am = fmaxf(group_max<EPL>(am), 1e-12f);
+        const float av = fmaxf(sqrt_rn(group_max<EPL>(vm)), 1e-12f);
+        quantize_mom<EPL>(m, am, mraw);
+        quantize_var<EPL>(r, av, vraw);
+        store_lane<1, EPL, FAST>(mraw, t.mom, first, n);
+        store_lane<1, EPL, FAST>(vraw, t.var, first, n);
+        if (live_group && (threadIdx.x & (32 / EPL - 1)) == 0) {                    // ref:2424-2434
             t.mom_scales[group] = f32_to_f16_bits(am);
             t.var_scales[group] = f32_to_f16_bits(av);
         }
     } else {
-        narrow_all<DT>(m, mraw);                                                 // ref:2435-2438
-        narrow_all<DT>(v, vraw);
-        store_lane<SB, FAST>(mraw, t.mom, first, n);
-        store_lane<SB, FAST>(vraw, t.var, first, n);
+        narrow_all<DT, EPL>(m, mraw);                                               // ref:2435-2438
+        narrow_all<DT, EPL>(v, vraw);
+        store_lane<SB, EPL, FAST>(mraw, t.mom, first, n);
+        store_lane<SB, EPL, FAST>(vraw, t.var, first, n);
     }
 }
-
 
 template <int DT, int ECCB, bool QUANT, bool DECOUPLED> struct AdamOp {
     using Hyper = AdamHyper;
     static constexpr bool kNeedsLut = QUANT;
+    static constexpr int kEpl = DTypeInfo<DT>::epl;
     template <bool FAST>
     __device__ __forceinline__ static void lane(const TensorPtrs& t, int64_t first, const Hyper& h, const float* lut) {
         adam_lane<DT, ECCB, QUANT, DECOUPLED, FAST>(t, first, h, lut);
@@ -117,24 +123,28 @@ template <int DT, int EB, bool Q> using AdamL2Op = fo::AdamOp<DT, EB, Q, false>;
 template <int DT, int EB, bool Q> using AdamWOp = fo::AdamOp<DT, EB, Q, true>;    // FlashAdamW: decay applied to the weights
 
 fo::AdamHyper make_adam_hyper(float lr, float beta1, float beta2, float eps, float wd, int step) {
-    // Scalars arrive as fp32 like the reference's kernel arguments; 1 - x is formed in fp32 (ref:2357-2364).
-    // beta^step is the correctly rounded fp32 power; the bias corrections are folded into two per-launch
-    // factors in double and rounded once.
     fo::AdamHyper h;
     h.b1 = beta1; h.one_m_b1 = 1.0f - beta1;
     h.b2 = beta2; h.one_m_b2 = 1.0f - beta2;
     h.wd = wd; h.one_m_wd = 1.0f - wd;
-    const float bc1 = 1.0f - (float)std::pow((double)beta1, (double)step);
-    const float bc2 = 1.0f - (float)std::pow((double)beta2, (double)step);
-    h.lr_over_bc1 = (float)((double)lr / (double)bc1);
-    h.rsqrt_bc2 = (float)(1.0 / std::sqrt((double)bc2));
-    h.eps = eps;
+    h.sqrt_b2_over_255 = (float)(std::sqrt((double)beta2) / 255.0);
+    // beta^step is the correctly rounded fp32 power, 1 - that is formed in fp32 (ref:2368-2369)
+    const double bc1 = (double)(1.0f - (float)std::pow((double)beta1, (double)step));
+    const double bc2 = (double)(1.0f - (float)std::pow((double)beta2, (double)step));
+    if (lr != 0.0f) {
+        h.den_scale = (float)(bc1 / ((double)lr * std::sqrt(bc2)));
+        h.den_bias = (float)((double)eps * bc1 / (double)lr);
+    } else {  // no update: the denominator is infinite whatever sqrt(v) is
+        h.den_scale = 0.0f;
+        h.den_bias = std::numeric_limits<float>::infinity();
+    }
     return h;
 }
 
 }  // namespace
 
 extern "C" {
+
 int fo_adam_step(void* mom, void* mom_scales, void* var, void* var_scales, void* param, const void* grad, void* ecc,
                  int64_t n, int dtype, int ecc_bytes, int quantized, float lr, float beta1, float beta2, float eps,
                  float weight_decay, int decoupled, int step, void* stream) {

@@ -1,7 +1,7 @@
 // Standalone group codec and ECC kernels for gfx950 with their C entry points: the cold-path companions of
 // the fused step kernels (state initialisation, uncompressed checkpoints, fp32 export/import of master
-// weights).  They share the lane layout of the step kernels (16 consecutive elements per lane, one 32-element
-// group per lane pair) and use correctly rounded division / square root, so that their output equals an IEEE
+// weights).  They share the access shape of the step kernels (fo_device.h) and use correctly rounded division /
+// square root, so that their output equals an IEEE
 // evaluation of the reference formulas operation by operation.
 //
 // "ref:" cites /root/reference/flashoptim/optimizers.py.
@@ -11,6 +11,8 @@
 
 namespace fo {
 
+constexpr int kCodecThreads = 256;
+
 struct CodecFlags {
     int is_signed, do_sqrt, softsign;
 };
@@ -18,121 +20,124 @@ struct CodecFlags {
 // ref:2610-2676 _triton_quantize_kernel
 template <int XDT, bool FAST>
 __device__ __forceinline__ void quantize_lane(const void* x, void* codes, uint16_t* scales, int64_t first, int64_t n, CodecFlags f) {
-    Pack<DTypeInfo<XDT>::bytes> xraw;
-    load_lane<DTypeInfo<XDT>::bytes, FAST>(xraw, x, first, n);
-    float v[kLaneElems];
+    constexpr int EPL = DTypeInfo<XDT>::epl;
+    Pack<DTypeInfo<XDT>::bytes, EPL> xraw;
+    load_lane<DTypeInfo<XDT>::bytes, EPL, FAST>(xraw, x, first, n);
+    float v[EPL];
     float am = 0.0f;
 #pragma unroll
-    for (int k = 0; k < kLaneElems; ++k) {
-        float t = widen<XDT>(xraw, k);
-        if (f.do_sqrt) t = sqrt_rn(t);                                   // ref:2650-2651
+    for (int k = 0; k < EPL; ++k) {
+        float t = widen<XDT, EPL>(xraw, k);
+        if (f.do_sqrt) t = sqrt_rn(t);                                      // ref:2650-2651
         v[k] = t;
         am = fmaxf(am, fabsf(t));
     }
-    am = fmaxf(fmaxf(am, pair_swap(am)), 1e-12f);                           // ref:2657-2658
+    am = fmaxf(group_max<EPL>(am), 1e-12f);                                 // ref:2657-2658
     const float out_max = f.is_signed ? 127.0f : 255.0f;
-    Pack<1> out;
+    u32 q[EPL];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) out.w[i] = 0;
-#pragma unroll
-    for (int k = 0; k < kLaneElems; ++k) {
-        const float nrm = div_rn(v[k], am);                              // ref:2661
+    for (int k = 0; k < EPL; ++k) {
+        const float nrm = div_rn(v[k], am);                                 // ref:2661
         const float t = f.softsign ? div_rn(2.0f * nrm, 1.0f + fabsf(nrm)) : nrm;   // ref:2664-2667
-        const float q = floorf(t * out_max + 0.5f);                         // ref:2670-2671
-        out.w[k / 4] |= ((u32)(int)q & 0xffu) << (8 * (k % 4));
+        q[k] = (u32)(int)floorf(t * out_max + 0.5f);                        // ref:2670-2671
     }
-    store_lane<1, FAST>(out, codes, first, n);
-    if ((FAST || first < n) && (threadIdx.x & 1) == 0) scales[first >> 5] = f32_to_f16_bits(am);   // ref:2675-2676
+    Pack<1, EPL> out;
+    pack_codes<1, EPL>(q, out);
+    store_lane<1, EPL, FAST>(out, codes, first, n);
+    if ((FAST || first < n) && (threadIdx.x & (32 / EPL - 1)) == 0) scales[first >> 5] = f32_to_f16_bits(am);   // ref:2675-2676
 }
 
 // ref:2541-2607 _triton_dequantize_kernel
 template <bool FAST>
 __device__ __forceinline__ void dequantize_lane(const void* codes, const uint16_t* scales, float* out, int64_t first, int64_t n, CodecFlags f) {
-    Pack<1> craw;
-    load_lane<1, FAST>(craw, codes, first, n);
+    constexpr int EPL = 4;
+    Pack<1, EPL> craw;
+    load_lane<1, EPL, FAST>(craw, codes, first, n);
     float scale = 1.0f;                                                     // ref:2577-2582 masked scales read 1.0
     if (FAST || first < n) scale = f16_bits_to_f32(scales[first >> 5]);
     const float in_max = f.is_signed ? 127.0f : 255.0f;
-    Pack<4> o;
+    Pack<4, EPL> o;
 #pragma unroll
-    for (int k = 0; k < kLaneElems; ++k) {
-        const u32 b = byte_of(craw, k);
+    for (int k = 0; k < EPL; ++k) {
+        const u32 b = byte_of<EPL>(craw, k);
         const float q = f.is_signed ? (float)(int8_t)b : (float)b;
-        const float t = div_rn(q, in_max);                               // ref:2591
-        const float nrm = f.softsign ? div_rn(t, 2.0f - fabsf(t)) : t;   // ref:2594-2597
+        const float t = div_rn(q, in_max);                                  // ref:2591
+        const float nrm = f.softsign ? div_rn(t, 2.0f - fabsf(t)) : t;      // ref:2594-2597
         float xv = nrm * scale;                                             // ref:2600
         if (f.do_sqrt) xv = xv * xv;                                        // ref:2603-2604
         o.w[k] = as_u32(xv);
     }
-    store_lane<4, FAST>(o, out, first, n);
+    store_lane<4, EPL, FAST>(o, out, first, n);
 }
 
 // ref:2779-2803 _reconstruct_fp32_kernel
 template <int DT, int ECCB, bool FAST>
 __device__ __forceinline__ void ecc_join_lane(const void* narrow, const void* ecc, float* out, int64_t first, int64_t n) {
-    Pack<DTypeInfo<DT>::bytes> nraw;
-    Pack<ECCB> eraw;
-    load_lane<DTypeInfo<DT>::bytes, FAST>(nraw, narrow, first, n);
-    load_lane<ECCB, FAST>(eraw, ecc, first, n);
-    Pack<4> o;
+    constexpr int EPL = 4;
+    Pack<DTypeInfo<DT>::bytes, EPL> nraw;
+    Pack<ECCB, EPL> eraw;
+    load_lane<DTypeInfo<DT>::bytes, EPL, FAST>(nraw, narrow, first, n);
+    load_lane<ECCB, EPL, FAST>(eraw, ecc, first, n);
+    Pack<4, EPL> o;
 #pragma unroll
-    for (int k = 0; k < kLaneElems; ++k) o.w[k] = as_u32(ecc_join<DT, ECCB>(widen<DT>(nraw, k), ecc_to_float<ECCB>(eraw, k)));
-    store_lane<4, FAST>(o, out, first, n);
+    for (int k = 0; k < EPL; ++k) o.w[k] = as_u32(ecc_join<DT, ECCB>(widen<DT, EPL>(nraw, k), ecc_to_float<ECCB, EPL>(eraw, k)));
+    store_lane<4, EPL, FAST>(o, out, first, n);
 }
 
 // ref:2806-2832 _compute_ecc_bits_kernel
 template <int DT, int ECCB, bool FAST>
 __device__ __forceinline__ void ecc_split_lane(const float* x, const void* narrow, void* ecc, int64_t first, int64_t n) {
-    Pack<4> xraw;
-    Pack<DTypeInfo<DT>::bytes> nraw;
-    load_lane<4, FAST>(xraw, x, first, n);
-    load_lane<DTypeInfo<DT>::bytes, FAST>(nraw, narrow, first, n);
-    u32 eb[kLaneElems];
+    constexpr int EPL = 4;
+    Pack<4, EPL> xraw;
+    Pack<DTypeInfo<DT>::bytes, EPL> nraw;
+    load_lane<4, EPL, FAST>(xraw, x, first, n);
+    load_lane<DTypeInfo<DT>::bytes, EPL, FAST>(nraw, narrow, first, n);
+    u32 eb[EPL];
 #pragma unroll
-    for (int k = 0; k < kLaneElems; ++k) eb[k] = ecc_split_bits<DT, ECCB>(as_f32(xraw.w[k]), widen<DT>(nraw, k));
-    Pack<ECCB> eout;
-    if constexpr (ECCB == 1) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) eout.w[i] = pack_bytes4(eb[4 * i], eb[4 * i + 1], eb[4 * i + 2], eb[4 * i + 3]);
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) eout.w[i] = pack_halves2(eb[2 * i], eb[2 * i + 1]);
-    }
-    store_lane<ECCB, FAST>(eout, ecc, first, n);
+    for (int k = 0; k < EPL; ++k) eb[k] = ecc_split_bits<DT, ECCB, true>(as_f32(xraw.w[k]), widen<DT, EPL>(nraw, k));
+    Pack<ECCB, EPL> eout;
+    pack_codes<ECCB, EPL>(eb, eout);
+    store_lane<ECCB, EPL, FAST>(eout, ecc, first, n);
 }
 
-// Tile loop shared by the four kernels: body(first, fast_tag) per lane.
-#define FO_TILE_LOOP(N, ALIGNED, CALL_FAST, CALL_SLOW)                                            \
+// Tile loop shared by the four kernels: blocks stride over 4096-element tiles, wavefronts over the tile's
+// sub-tiles of 64 x EPL elements; `first` is the lane's first element.
+#define FO_TILE_LOOP(N, EPL_, ALIGNED, CALL_FAST, CALL_SLOW)                                      \
     {                                                                                             \
+        constexpr int kSub_ = 64 * (EPL_);                                                        \
+        const int lane_ = threadIdx.x & 63, wave_ = threadIdx.x >> 6;                             \
         const int64_t n_tiles_ = ((N) + kTileElems - 1) / kTileElems;                             \
         for (int64_t tile_ = blockIdx.x; tile_ < n_tiles_; tile_ += gridDim.x) {                  \
             const int64_t base_ = tile_ * (int64_t)kTileElems;                                    \
-            const int64_t first = base_ + (int64_t)threadIdx.x * kLaneElems;                      \
-            if ((ALIGNED) && base_ + kTileElems <= (N)) { CALL_FAST; } else { CALL_SLOW; }        \
+            const bool fast_ = (ALIGNED) && base_ + kTileElems <= (N);                            \
+            for (int s_ = wave_; s_ < kTileElems / kSub_; s_ += kCodecThreads / 64) {             \
+                const int64_t first = base_ + s_ * kSub_ + lane_ * (EPL_);                        \
+                if (fast_) { CALL_FAST; } else { CALL_SLOW; }                                     \
+            }                                                                                     \
         }                                                                                         \
     }
 
 template <int XDT>
-__global__ __launch_bounds__(kBlockThreads) void quantize_kernel(const void* x, void* codes, uint16_t* scales, int64_t n, CodecFlags f) {
+__global__ __launch_bounds__(kCodecThreads) void quantize_kernel(const void* x, void* codes, uint16_t* scales, int64_t n, CodecFlags f) {
     const bool aligned = ((((uintptr_t)x) | ((uintptr_t)codes)) & 15u) == 0;
-    FO_TILE_LOOP(n, aligned, (quantize_lane<XDT, true>(x, codes, scales, first, n, f)), (quantize_lane<XDT, false>(x, codes, scales, first, n, f)))
+    FO_TILE_LOOP(n, DTypeInfo<XDT>::epl, aligned, (quantize_lane<XDT, true>(x, codes, scales, first, n, f)), (quantize_lane<XDT, false>(x, codes, scales, first, n, f)))
 }
 
-__global__ __launch_bounds__(kBlockThreads) void dequantize_kernel(const void* codes, const uint16_t* scales, float* out, int64_t n, CodecFlags f) {
+__global__ __launch_bounds__(kCodecThreads) void dequantize_kernel(const void* codes, const uint16_t* scales, float* out, int64_t n, CodecFlags f) {
     const bool aligned = ((((uintptr_t)out) | ((uintptr_t)codes)) & 15u) == 0;
-    FO_TILE_LOOP(n, aligned, (dequantize_lane<true>(codes, scales, out, first, n, f)), (dequantize_lane<false>(codes, scales, out, first, n, f)))
+    FO_TILE_LOOP(n, 4, aligned, (dequantize_lane<true>(codes, scales, out, first, n, f)), (dequantize_lane<false>(codes, scales, out, first, n, f)))
 }
 
 template <int DT, int ECCB>
-__global__ __launch_bounds__(kBlockThreads) void ecc_join_kernel(const void* narrow, const void* ecc, float* out, int64_t n) {
+__global__ __launch_bounds__(kCodecThreads) void ecc_join_kernel(const void* narrow, const void* ecc, float* out, int64_t n) {
     const bool aligned = ((((uintptr_t)narrow) | ((uintptr_t)ecc) | ((uintptr_t)out)) & 15u) == 0;
-    FO_TILE_LOOP(n, aligned, (ecc_join_lane<DT, ECCB, true>(narrow, ecc, out, first, n)), (ecc_join_lane<DT, ECCB, false>(narrow, ecc, out, first, n)))
+    FO_TILE_LOOP(n, 4, aligned, (ecc_join_lane<DT, ECCB, true>(narrow, ecc, out, first, n)), (ecc_join_lane<DT, ECCB, false>(narrow, ecc, out, first, n)))
 }
 
 template <int DT, int ECCB>
-__global__ __launch_bounds__(kBlockThreads) void ecc_split_kernel(const float* x, const void* narrow, void* ecc, int64_t n) {
+__global__ __launch_bounds__(kCodecThreads) void ecc_split_kernel(const float* x, const void* narrow, void* ecc, int64_t n) {
     const bool aligned = ((((uintptr_t)narrow) | ((uintptr_t)ecc) | ((uintptr_t)x)) & 15u) == 0;
-    FO_TILE_LOOP(n, aligned, (ecc_split_lane<DT, ECCB, true>(x, narrow, ecc, first, n)), (ecc_split_lane<DT, ECCB, false>(x, narrow, ecc, first, n)))
+    FO_TILE_LOOP(n, 4, aligned, (ecc_split_lane<DT, ECCB, true>(x, narrow, ecc, first, n)), (ecc_split_lane<DT, ECCB, false>(x, narrow, ecc, first, n)))
 }
 
 }  // namespace fo
@@ -160,7 +165,7 @@ int fo_quantize(const void* x, int x_dtype, void* codes, void* scales, int64_t n
     const int cus = compute_units();
     if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
     const fo::CodecFlags f{is_signed ? 1 : 0, do_sqrt ? 1 : 0, softsign ? 1 : 0};
-    const dim3 grid(grid_for(n, cus)), block(fo::kBlockThreads);
+    const dim3 grid(grid_for(n, cus)), block(fo::kCodecThreads);
     hipStream_t s = (hipStream_t)stream;
     switch (x_dtype) {
         case FO_F32: hipLaunchKernelGGL(fo::quantize_kernel<fo::DT_F32>, grid, block, 0, s, x, codes, (uint16_t*)scales, n, f); break;
@@ -179,7 +184,7 @@ int fo_dequantize(const void* codes, const void* scales, float* out, int64_t n, 
     const int cus = compute_units();
     if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
     const fo::CodecFlags f{is_signed ? 1 : 0, do_sqrt ? 1 : 0, softsign ? 1 : 0};
-    hipLaunchKernelGGL(fo::dequantize_kernel, dim3(grid_for(n, cus)), dim3(fo::kBlockThreads), 0, (hipStream_t)stream, codes,
+    hipLaunchKernelGGL(fo::dequantize_kernel, dim3(grid_for(n, cus)), dim3(fo::kCodecThreads), 0, (hipStream_t)stream, codes,
                        (const uint16_t*)scales, out, n, f);
     return check_hip(hipGetLastError(), "dequantize kernel launch");
 }
@@ -204,7 +209,7 @@ int fo_ecc_join(const void* narrow, int narrow_dtype, const void* ecc, int ecc_b
     if (((uintptr_t)narrow & 1) || ((uintptr_t)out & 3) || (ecc_bytes == 2 && ((uintptr_t)ecc & 1))) return fail(FO_ERR_INVALID_ARGUMENT, "pointer not aligned to its element size");
     const int cus = compute_units();
     if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
-    const dim3 grid(grid_for(n, cus)), block(fo::kBlockThreads);
+    const dim3 grid(grid_for(n, cus)), block(fo::kCodecThreads);
     hipStream_t s = (hipStream_t)stream;
     FO_ECC_DISPATCH(ecc_join_kernel, narrow, ecc, out, n)
     return check_hip(hipGetLastError(), "ecc join kernel launch");
@@ -216,7 +221,7 @@ int fo_ecc_split(const float* x, const void* narrow, int narrow_dtype, void* ecc
     if (((uintptr_t)narrow & 1) || ((uintptr_t)x & 3) || (ecc_bytes == 2 && ((uintptr_t)ecc & 1))) return fail(FO_ERR_INVALID_ARGUMENT, "pointer not aligned to its element size");
     const int cus = compute_units();
     if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
-    const dim3 grid(grid_for(n, cus)), block(fo::kBlockThreads);
+    const dim3 grid(grid_for(n, cus)), block(fo::kCodecThreads);
     hipStream_t s = (hipStream_t)stream;
     FO_ECC_DISPATCH(ecc_split_kernel, x, narrow, ecc, n)
     return check_hip(hipGetLastError(), "ecc split kernel launch");

@@ -6,12 +6,15 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 
 namespace fo {
 
+constexpr int kCopyThreads = 256;
+
 // plain copy with the same access shape; calibrates byte counters and shows the attainable streaming rate
-__global__ __launch_bounds__(kBlockThreads) void copy_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, int64_t n_vec) {
-    for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < n_vec; i += (int64_t)gridDim.x * kBlockThreads)
+__global__ __launch_bounds__(kCopyThreads) void copy_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, int64_t n_vec) {
+    for (int64_t i = (int64_t)blockIdx.x * kCopyThreads + threadIdx.x; i < n_vec; i += (int64_t)gridDim.x * kCopyThreads)
         __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
@@ -37,6 +40,15 @@ int check_hip(hipError_t e, const char* what) {
 }
 
 const char* last_error() { return g_err; }
+
+int tiles_per_block() {
+    static const int value = [] {
+        const char* e = getenv("FO_TILES_PER_BLOCK");
+        const int v = e ? atoi(e) : 0;
+        return (v >= 1 && v <= 1024) ? v : 4;
+    }();
+    return value;
+}
 
 int compute_units() {
     static thread_local int cached_dev = -1, cached_cus = 0;
@@ -106,9 +118,9 @@ int fo_copy_bytes(void* dst, const void* src, int64_t n_bytes, void* stream) {
     const int cus = compute_units();
     if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
     const int64_t n_vec = n_bytes / 16;
-    const int64_t want = (n_vec + fo::kBlockThreads - 1) / fo::kBlockThreads;
+    const int64_t want = (n_vec + fo::kCopyThreads - 1) / fo::kCopyThreads;
     const int64_t cap = (int64_t)cus * kBlocksPerCu * 2;
-    hipLaunchKernelGGL(fo::copy_kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(fo::kBlockThreads), 0, (hipStream_t)stream,
+    hipLaunchKernelGGL(fo::copy_kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(fo::kCopyThreads), 0, (hipStream_t)stream,
                        (fo::u32x4*)dst, (const fo::u32x4*)src, n_vec);
     return check_hip(hipGetLastError(), "copy kernel launch");
 }

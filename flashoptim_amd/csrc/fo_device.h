@@ -2,6 +2,14 @@
 // narrowing, the ECC join/split and the 8-bit group codec.  Everything here is wave64 CDNA code; the file is
 // compiled with -ffp-contract=off, so a fused multiply-add happens only where fmaf() is written.
 //
+// Access shape.  A wavefront works on one "sub-tile" at a time: 64 lanes x EPL consecutive elements, where
+// EPL = 16 bytes / sizeof(parameter element) (8 for bf16/fp16, 4 for fp32).  Lane l owns elements
+// [l*EPL, (l+1)*EPL) of the sub-tile, so every parameter/gradient access is one 128-bit load or store per
+// lane and consecutive lanes touch consecutive 16-byte pieces: each wave-level instruction covers 1 KiB of
+// contiguous memory.  The 1-byte streams (codes, int8 ECC) move EPL bytes per lane (64- or 32-bit accesses,
+// again contiguous across the wave).  A 32-element quantisation group is 32/EPL neighbouring lanes (a DPP
+// quad for bf16/fp16), so the group absmax needs no LDS.
+//
 // "ref:" cites /root/reference/flashoptim/optimizers.py.
 #pragma once
 
@@ -11,16 +19,15 @@
 namespace fo {
 
 typedef uint32_t u32;
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
 typedef u32 u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kGroup = 32;                               // ref:1549, 2219: quantisation group
-constexpr int kLaneElems = 16;                           // contiguous elements owned by one lane
-constexpr int kBlockThreads = 256;                       // 4 wavefronts
-constexpr int kTileElems = kLaneElems * kBlockThreads;   // 4096 elements = 128 groups per block iteration
-constexpr float kMagic = 12582912.0f;                    // 1.5 * 2^23: x + kMagic leaves rne(x) in the low mantissa bits
+constexpr int kGroup = 32;             // ref:1549, 2219: quantisation group
+constexpr int kTileElems = 4096;       // unit of the multi-tensor chunk table (FO_TILE_ELEMS)
+constexpr float kMagic = 12582912.0f;  // 1.5 * 2^23: x + kMagic leaves rne(x) in the low mantissa bits
 
 enum { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2 };
 
@@ -34,52 +41,63 @@ __device__ __forceinline__ float as_f32(u32 u) { return __builtin_bit_cast(float
 __device__ __forceinline__ u32 as_u32(float f) { return __builtin_bit_cast(u32, f); }
 
 template <int DT> struct DTypeInfo;
-template <> struct DTypeInfo<DT_F32> { static constexpr int bytes = 4, mant = 23; };
-template <> struct DTypeInfo<DT_BF16> { static constexpr int bytes = 2, mant = 7; };
-template <> struct DTypeInfo<DT_F16> { static constexpr int bytes = 2, mant = 10; };
+template <> struct DTypeInfo<DT_F32> { static constexpr int bytes = 4, mant = 23, epl = 4; };
+template <> struct DTypeInfo<DT_BF16> { static constexpr int bytes = 2, mant = 7, epl = 8; };
+template <> struct DTypeInfo<DT_F16> { static constexpr int bytes = 2, mant = 10, epl = 8; };
 
 // ------------------------------------------------------------------------------------------------
-// Lane-private packed storage: 16 elements of EB bytes each, kept as the dwords that travel to memory.
+// Lane-private packed storage: EPL elements of EB bytes each (4, 8 or 16 bytes in total), kept as the
+// dwords that travel to memory.  EB == 0 is an absent stream.
 // ------------------------------------------------------------------------------------------------
-template <int EB> struct Pack {
-    static constexpr int kDwords = EB * kLaneElems / 4;  // 4, 8 or 16
+template <int EB, int EPL> struct Pack {
+    static constexpr int kBytes = EB * EPL;
+    static constexpr int kDwords = kBytes / 4;
+    static_assert(kBytes == 4 || kBytes == 8 || kBytes == 16, "a lane moves 4, 8 or 16 bytes per stream");
     u32 w[kDwords];
 };
-template <> struct Pack<0> {
+template <int EPL> struct Pack<0, EPL> {
+    static constexpr int kBytes = 0;
     static constexpr int kDwords = 0;
     u32 w[1];
 };
 
-// Fast path: the lane's 16 elements are in range and the base pointer is 16-byte aligned, so the lane moves
-// 16*EB contiguous bytes with 128-bit accesses.  The streams are touched once per step: non-temporal hint.
-template <int EB>
-__device__ __forceinline__ void load_vec(Pack<EB>& d, const void* base, int64_t first) {
-    const u32x4* p = reinterpret_cast<const u32x4*>(static_cast<const char*>(base) + first * EB);
-#pragma unroll
-    for (int i = 0; i < Pack<EB>::kDwords / 4; ++i) {
-        u32x4 v = __builtin_nontemporal_load(p + i);
-        d.w[4 * i + 0] = v.x; d.w[4 * i + 1] = v.y; d.w[4 * i + 2] = v.z; d.w[4 * i + 3] = v.w;
+// Fast path: all EPL elements are in range and the address is aligned to the access size; one vector access
+// per lane.  Every stream is touched exactly once per step, hence the non-temporal hint.
+template <int EB, int EPL>
+__device__ __forceinline__ void load_vec(Pack<EB, EPL>& d, const void* base, int64_t first) {
+    const char* p = static_cast<const char*>(base) + first * EB;
+    if constexpr (Pack<EB, EPL>::kBytes == 16) {
+        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+        d.w[0] = v.x; d.w[1] = v.y; d.w[2] = v.z; d.w[3] = v.w;
+    } else if constexpr (Pack<EB, EPL>::kBytes == 8) {
+        const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+        d.w[0] = v.x; d.w[1] = v.y;
+    } else {
+        d.w[0] = __builtin_nontemporal_load(reinterpret_cast<const u32*>(p));
     }
 }
-template <int EB>
-__device__ __forceinline__ void store_vec(const Pack<EB>& d, void* base, int64_t first) {
-    u32x4* p = reinterpret_cast<u32x4*>(static_cast<char*>(base) + first * EB);
-#pragma unroll
-    for (int i = 0; i < Pack<EB>::kDwords / 4; ++i) {
-        u32x4 v;
-        v.x = d.w[4 * i + 0]; v.y = d.w[4 * i + 1]; v.z = d.w[4 * i + 2]; v.w = d.w[4 * i + 3];
-        __builtin_nontemporal_store(v, p + i);
+template <int EB, int EPL>
+__device__ __forceinline__ void store_vec(const Pack<EB, EPL>& d, void* base, int64_t first) {
+    char* p = static_cast<char*>(base) + first * EB;
+    if constexpr (Pack<EB, EPL>::kBytes == 16) {
+        u32x4 v; v.x = d.w[0]; v.y = d.w[1]; v.z = d.w[2]; v.w = d.w[3];
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+    } else if constexpr (Pack<EB, EPL>::kBytes == 8) {
+        u32x2 v; v.x = d.w[0]; v.y = d.w[1];
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
+    } else {
+        __builtin_nontemporal_store(d.w[0], reinterpret_cast<u32*>(p));
     }
 }
 
 // Guarded path (tensor tails, unaligned views): element-wise accesses, out-of-range elements read as zero and
 // are never written (ref:1625-1630, 2296-2301 masked loads with other=0).
-template <int EB>
-__device__ __forceinline__ void load_guarded(Pack<EB>& d, const void* base, int64_t first, int64_t n) {
+template <int EB, int EPL>
+__device__ __forceinline__ void load_guarded(Pack<EB, EPL>& d, const void* base, int64_t first, int64_t n) {
 #pragma unroll
-    for (int i = 0; i < Pack<EB>::kDwords; ++i) d.w[i] = 0;
+    for (int i = 0; i < Pack<EB, EPL>::kDwords; ++i) d.w[i] = 0;
 #pragma unroll
-    for (int k = 0; k < kLaneElems; ++k) {
+    for (int k = 0; k < EPL; ++k) {
         const int64_t idx = first + k;
         if (idx < n) {
             if constexpr (EB == 1) d.w[k / 4] |= (u32) static_cast<const uint8_t*>(base)[idx] << (8 * (k % 4));
@@ -88,10 +106,10 @@ __device__ __forceinline__ void load_guarded(Pack<EB>& d, const void* base, int6
         }
     }
 }
-template <int EB>
-__device__ __forceinline__ void store_guarded(const Pack<EB>& d, void* base, int64_t first, int64_t n) {
+template <int EB, int EPL>
+__device__ __forceinline__ void store_guarded(const Pack<EB, EPL>& d, void* base, int64_t first, int64_t n) {
 #pragma unroll
-    for (int k = 0; k < kLaneElems; ++k) {
+    for (int k = 0; k < EPL; ++k) {
         const int64_t idx = first + k;
         if (idx < n) {
             if constexpr (EB == 1) static_cast<uint8_t*>(base)[idx] = (uint8_t)(d.w[k / 4] >> (8 * (k % 4)));
@@ -100,23 +118,23 @@ __device__ __forceinline__ void store_guarded(const Pack<EB>& d, void* base, int
         }
     }
 }
-template <int EB, bool FAST>
-__device__ __forceinline__ void load_lane(Pack<EB>& d, const void* base, int64_t first, int64_t n) {
+template <int EB, int EPL, bool FAST>
+__device__ __forceinline__ void load_lane(Pack<EB, EPL>& d, const void* base, int64_t first, int64_t n) {
     if constexpr (EB > 0) {
-        if constexpr (FAST) load_vec<EB>(d, base, first); else load_guarded<EB>(d, base, first, n);
+        if constexpr (FAST) load_vec<EB, EPL>(d, base, first); else load_guarded<EB, EPL>(d, base, first, n);
     }
 }
-template <int EB, bool FAST>
-__device__ __forceinline__ void store_lane(const Pack<EB>& d, void* base, int64_t first, int64_t n) {
+template <int EB, int EPL, bool FAST>
+__device__ __forceinline__ void store_lane(const Pack<EB, EPL>& d, void* base, int64_t first, int64_t n) {
     if constexpr (EB > 0) {
-        if constexpr (FAST) store_vec<EB>(d, base, first); else store_guarded<EB>(d, base, first, n);
+        if constexpr (FAST) store_vec<EB, EPL>(d, base, first); else store_guarded<EB, EPL>(d, base, first, n);
     }
 }
 
 // ------------------------------------------------------------------------------------------------
 // widening / narrowing of the parameter dtype
 // ------------------------------------------------------------------------------------------------
-template <int DT> __device__ __forceinline__ float widen(const Pack<DTypeInfo<DT>::bytes>& d, int k) {
+template <int DT, int EPL> __device__ __forceinline__ float widen(const Pack<DTypeInfo<DT>::bytes, EPL>& d, int k) {
     if constexpr (DT == DT_F32) return as_f32(d.w[k]);
     if constexpr (DT == DT_BF16) return as_f32((k & 1) ? (d.w[k / 2] & 0xffff0000u) : (d.w[k / 2] << 16));
     if constexpr (DT == DT_F16) {
@@ -127,8 +145,8 @@ template <int DT> __device__ __forceinline__ float widen(const Pack<DTypeInfo<DT
 
 // Round to nearest even into the parameter dtype (ref:2377 param.to(PARAM_DTYPE)); writes elements k, k+1
 // and returns them widened back.  bf16 pairs use the gfx950 packed convert.
-template <int DT>
-__device__ __forceinline__ void narrow_pair(Pack<DTypeInfo<DT>::bytes>& d, int k, float a, float b, float& wa, float& wb) {
+template <int DT, int EPL>
+__device__ __forceinline__ void narrow_pair(Pack<DTypeInfo<DT>::bytes, EPL>& d, int k, float a, float b, float& wa, float& wb) {
     if constexpr (DT == DT_F32) {
         d.w[k] = as_u32(a); d.w[k + 1] = as_u32(b); wa = a; wb = b;
     }
@@ -150,16 +168,17 @@ template <int ECCB> struct EccInfo;
 template <> struct EccInfo<1> { static constexpr float max_val = 127.0f; };      // ref:1521
 template <> struct EccInfo<2> { static constexpr float max_val = 32767.0f; };    // ref:1523
 
-// Biased exponent field of the narrow value given its widened fp32 bits, with zero/subnormal mapped to the
-// smallest normal exponent (ref:2704-2712).  bf16 shares fp32's field; fp16's is recovered from the fp32 one
-// (an fp16 subnormal widens to an fp32 normal with exponent < -14, which the max() maps back to -14).
-template <int DT> __device__ __forceinline__ int narrow_exp_field(float widened) {
-    const int e = (int)((as_u32(widened) >> 23) & 0xffu);
-    if constexpr (DT == DT_F16) return max(e, 127 - 14);
-    return max(e, 1);
+// fp32 bit pattern of 2^E, E = unbiased exponent of the narrow value with zero/subnormal mapped to the
+// smallest normal exponent (ref:2704-2712), given the value widened to fp32.  bf16 shares fp32's exponent
+// field; an fp16 subnormal widens to an fp32 normal below 2^-14, which the lower clamp maps back to -14.
+// The upper clamp keeps inf/NaN inputs from producing an infinite scale.
+template <int DT> __device__ __forceinline__ u32 pow2_of_exponent_bits(float widened) {
+    constexpr u32 lo = (DT == DT_F16) ? ((127u - 14u) << 23) : (1u << 23);
+    const u32 e = as_u32(widened) & 0x7f800000u;
+    return min(max(e, lo), 254u << 23);
 }
 
-template <int ECCB> __device__ __forceinline__ float ecc_to_float(const Pack<ECCB>& d, int k) {
+template <int ECCB, int EPL> __device__ __forceinline__ float ecc_to_float(const Pack<ECCB, EPL>& d, int k) {
     if constexpr (ECCB == 1) return (float)(int8_t)(d.w[k / 4] >> (8 * (k % 4)));
     if constexpr (ECCB == 2) return (float)(int16_t)(d.w[k / 2] >> (16 * (k % 2)));
     return 0.0f;
@@ -168,15 +187,13 @@ template <int ECCB> __device__ __forceinline__ float ecc_to_float(const Pack<ECC
 // x_narrow + (ecc / MAX) * 2^(E - mant - 1) with the product and the sum fused (ref:2767-2776; the reference
 // compiles with FP fusion, and its invariants test only passes with the fused form).
 //   ecc / MAX is formed exactly rounded as fma(e, K_hi, e * K_lo) with K_hi + K_lo = 2^-(mant+1) / MAX to
-//   well beyond fp32 precision (checked exhaustively over every int8 / int16 value on the host);
-//   2^E comes straight from the exponent field; inf/NaN inputs (field 255) are clamped to 254.
+//   well beyond fp32 precision (checked exhaustively over every int8 / int16 value on the host).
 template <int DT, int ECCB> __device__ __forceinline__ float ecc_join(float widened, float ecc) {
     constexpr double k = 1.0 / ((double)EccInfo<ECCB>::max_val * (double)(1 << (DTypeInfo<DT>::mant + 1)));
     constexpr float k_hi = (float)k;
     constexpr float k_lo = (float)(k - (double)k_hi);
     const float c = fmaf(ecc, k_hi, ecc * k_lo);
-    const int e = min(narrow_exp_field<DT>(widened), 254);
-    return fmaf(c, as_f32((u32)e << 23), widened);
+    return fmaf(c, as_f32(pow2_of_exponent_bits<DT>(widened)), widened);
 }
 
 // Signed fraction of half an ulp of the NEW narrow value, scaled to +-MAX and rounded half away from zero
@@ -186,20 +203,21 @@ template <int DT, int ECCB> __device__ __forceinline__ float ecc_join(float wide
 //   bf16 with an int8 code: p - narrow is exact and a multiple of 2^-16 half-ulps, so en * 127 fits 24 bits and
 //   is exact; the only tie that can occur is +-63.5, where half-even and half-away agree.  One fma against
 //   1.5 * 2^23 then leaves the rounded integer in the low mantissa bits.
-template <int DT, int ECCB> __device__ __forceinline__ u32 ecc_split_bits(float p, float widened) {
+//   CLAMP = false is for callers whose narrow value IS the round-to-nearest of p (|en| <= 1 by construction).
+template <int DT, int ECCB, bool CLAMP> __device__ __forceinline__ u32 ecc_split_bits(float p, float widened) {
     const float err = p - widened;
-    const int nls = (DTypeInfo<DT>::mant + 1 + 127) - narrow_exp_field<DT>(widened);
-    const float en = __builtin_amdgcn_ldexpf(err, nls);
-    const float cl = __builtin_amdgcn_fmed3f(en, -1.0f, 1.0f);
+    const int nls = (DTypeInfo<DT>::mant + 1 + 127) - (int)(pow2_of_exponent_bits<DT>(widened) >> 23);
+    float en = __builtin_amdgcn_ldexpf(err, nls);
+    if constexpr (CLAMP) en = __builtin_amdgcn_fmed3f(en, -1.0f, 1.0f);
     if constexpr (DT == DT_BF16 && ECCB == 1) {
-        return as_u32(fmaf(cl, EccInfo<ECCB>::max_val, kMagic));
+        return as_u32(fmaf(en, EccInfo<ECCB>::max_val, kMagic));
     } else {
-        const float sc = cl * EccInfo<ECCB>::max_val;
+        const float sc = en * EccInfo<ECCB>::max_val;
         return (u32)(int)(sc + __builtin_copysignf(0.5f, sc));
     }
 }
 
-// Gathers the low byte (or low half) of consecutive magic-rounded words into packed storage.
+// Gathers the low byte (or low half) of consecutive code words into packed storage.
 __device__ __forceinline__ u32 pack_bytes4(u32 a, u32 b, u32 c, u32 d) {
     const u32 lo = __builtin_amdgcn_perm(b, a, 0x0c0c0400u);  // a.b0 | b.b0 << 8
     const u32 hi = __builtin_amdgcn_perm(d, c, 0x04000c0cu);  // c.b0 << 16 | d.b0 << 24
@@ -207,46 +225,67 @@ __device__ __forceinline__ u32 pack_bytes4(u32 a, u32 b, u32 c, u32 d) {
 }
 __device__ __forceinline__ u32 pack_halves2(u32 a, u32 b) { return __builtin_amdgcn_perm(b, a, 0x05040100u); }
 
+template <int EB, int EPL> __device__ __forceinline__ void pack_codes(const u32 (&c)[EPL], Pack<EB, EPL>& out) {
+    if constexpr (EB == 1) {
+#pragma unroll
+        for (int i = 0; i < EPL / 4; ++i) out.w[i] = pack_bytes4(c[4 * i], c[4 * i + 1], c[4 * i + 2], c[4 * i + 3]);
+    }
+    if constexpr (EB == 2) {
+#pragma unroll
+        for (int i = 0; i < EPL / 2; ++i) out.w[i] = pack_halves2(c[2 * i], c[2 * i + 1]);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // 8-bit group codec pieces used by the fused kernels
 // ------------------------------------------------------------------------------------------------
 
-// value of lane (id ^ 1): the two lanes that share a 32-element group are neighbours
-__device__ __forceinline__ float pair_swap(float x) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xf, 0xf, true));
+template <int CTRL> __device__ __forceinline__ float dpp_move(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
 }
 
-// rn(q / 255) for q in 0..255, exact: fma(q, hi, q*lo) with hi+lo = 1/255 (checked exhaustively on the host)
-__device__ __forceinline__ float code255_to_unit(float q) {
-    constexpr float hi = (float)(1.0 / 255.0);
-    constexpr float lo = (float)(1.0 / 255.0 - (double)hi);
-    return fmaf(q, hi, q * lo);
+// max over the 32/EPL neighbouring lanes that share one quantisation group; every lane gets the result
+template <int EPL> __device__ __forceinline__ float group_max(float x) {
+    x = fmaxf(x, dpp_move<0xB1>(x));  // quad_perm [1,0,3,2]
+    x = fmaxf(x, dpp_move<0x4E>(x));  // quad_perm [2,3,0,1]: now the max of each aligned group of 4 lanes
+    if constexpr (EPL == 4) x = fmaxf(x, dpp_move<0x141>(x));  // row_half_mirror: swaps the two quads of each 8 lanes
+    return x;
 }
 
-// Dequantised first-moment magnitude for signed code byte b, before the scale: (q/127) / (2 - |q/127|)
-// (ref:2332-2336), IEEE-rounded at each step.  Filled once per block into a bank-replicated LDS table.
-__device__ __forceinline__ float softsign_inverse_of_code(int q) {
-    const float y = div_rn((float)q, 127.0f);
-    return div_rn(y, 2.0f - fabsf(y));
-}
+// Dequantised first-moment magnitude for signed code byte b, before the scale:
+// (q/127) / (2 - |q/127|) (ref:2332-2336), each operation correctly rounded.  Evaluated by the compiler.
+struct SoftsignTable {
+    float v[256];
+    constexpr SoftsignTable() : v() {
+        for (int b = 0; b < 256; ++b) {
+            const int q = b < 128 ? b : b - 256;
+            const float y = (float)q / 127.0f;
+            const float a = y < 0.0f ? -y : y;
+            v[b] = y / (2.0f - a);
+        }
+    }
+};
+__device__ const SoftsignTable kSoftsignTable = SoftsignTable();
 
-constexpr int kLutFloats = 256 * 32;  // 32 KiB: entry for code byte b and lane l lives at [b*32 + (l & 31)]
-
-// One thread per code value writes its 32 bank copies, so later lookups never conflict: lane l always reads
-// bank l & 31 whatever its code is.
-__device__ __forceinline__ void build_softsign_lut(float* lut) {
-    const int b = threadIdx.x;  // blockDim.x == 256
-    const float v = softsign_inverse_of_code((int)(int8_t)b);
-    float4 v4 = make_float4(v, v, v, v);
-    float4* row = reinterpret_cast<float4*>(lut + b * 32);
+// The table lives in LDS during a kernel.  REPL copies per entry; a lane uses copy (lane % REPL).
+// REPL = 32 gives every lane its own bank (entry b, lane l at [b*32 + (l & 31)]): no bank conflicts.
+template <int REPL> struct Lut {
+    static constexpr int kFloats = 256 * REPL;
+    __device__ __forceinline__ static void build(float* lut) {
+        for (int b = threadIdx.x; b < 256; b += blockDim.x) {
+            const float v = kSoftsignTable.v[b];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) row[i] = v4;
-    __syncthreads();
-}
+            for (int i = 0; i < REPL; ++i) lut[b * REPL + i] = v;
+        }
+        __syncthreads();
+    }
+    __device__ __forceinline__ static const float* lane_base(const float* lut) { return lut + (threadIdx.x & (REPL - 1)); }
+    __device__ __forceinline__ static float lookup(const float* lane_lut, u32 byte) { return lane_lut[byte * REPL]; }
+};
 
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }  // RTNE
 
-__device__ __forceinline__ u32 byte_of(const Pack<1>& d, int k) { return (d.w[k / 4] >> (8 * (k % 4))) & 0xffu; }
+template <int EPL> __device__ __forceinline__ u32 byte_of(const Pack<1, EPL>& d, int k) { return (d.w[k / 4] >> (8 * (k % 4))) & 0xffu; }
 
 }  // namespace fo

@@ -15,7 +15,12 @@ int check_hip(hipError_t e, const char* what);
 int compute_units();
 const char* last_error();
 
-constexpr int kBlocksPerCu = 8;           // persistent-grid cap: blocks per compute unit
-constexpr int kDefaultTilesPerChunk = 8;  // multi-tensor work item = 8 tiles = 32768 elements
+// Tiles (4096 elements each) a block of the single-tensor kernels walks before it retires.  Small enough that
+// the launch is one pass of many short-lived blocks, large enough to amortise the per-block table set-up.
+// FO_TILES_PER_BLOCK in the environment overrides it (read once; for tuning).
+int tiles_per_block();
+
+constexpr int kBlocksPerCu = 8;           // grid cap of the cold-path kernels: blocks per compute unit
+constexpr int kDefaultTilesPerChunk = 4;  // multi-tensor work item = 4 tiles = 16384 elements
 
 }  // namespace fo_host

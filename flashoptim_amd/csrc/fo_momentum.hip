@@ -16,55 +16,55 @@ struct MomentumHyper {
 };
 
 template <int DT, int ECCB, bool QUANT, int KIND, bool FAST>
-__device__ __forceinline__ void momentum_lane(const TensorPtrs& t, int64_t first, const MomentumHyper& h,
-                                              const float* lut_lane) {
+__device__ __forceinline__ void momentum_lane(const TensorPtrs& t, int64_t first, const MomentumHyper& h, const float* lut_lane) {
+    constexpr int EPL = DTypeInfo<DT>::epl;
     constexpr int PB = DTypeInfo<DT>::bytes;
     constexpr int SB = (KIND == KIND_PLAIN) ? 0 : (QUANT ? 1 : PB);
     const int64_t n = t.n;
 
-    Pack<PB> praw, graw;
-    Pack<ECCB> eraw;
-    Pack<SB> mraw;
-    load_lane<PB, FAST>(graw, t.grad, first, n);
-    load_lane<PB, FAST>(praw, t.param, first, n);
-    load_lane<ECCB, FAST>(eraw, t.ecc, first, n);
-    load_lane<SB, FAST>(mraw, t.mom, first, n);
+    Pack<PB, EPL> praw, graw;
+    Pack<ECCB, EPL> eraw;
+    Pack<SB, EPL> mraw;
+    load_lane<PB, EPL, FAST>(graw, t.grad, first, n);
+    load_lane<PB, EPL, FAST>(praw, t.param, first, n);
+    load_lane<ECCB, EPL, FAST>(eraw, t.ecc, first, n);
+    load_lane<SB, EPL, FAST>(mraw, t.mom, first, n);
     const bool live_group = FAST || first < n;
     const int64_t group = first >> 5;
     float sm = 1.0f;
     if constexpr (QUANT && KIND != KIND_PLAIN) {
-        if (live_group) sm = f16_bits_to_f32(t.mom_scales[group]);               // ref:1645-1646
+        if (live_group) sm = f16_bits_to_f32(t.mom_scales[group]);                  // ref:1645-1646
     }
 
-    float p[kLaneElems], m[kLaneElems];
-    read_master<DT, ECCB>(p, praw, eraw);
+    float p[EPL], m[EPL];
+    read_master<DT, ECCB, EPL>(p, praw, eraw);
 
     float am = 0.0f;
 #pragma unroll
-    for (int k = 0; k < kLaneElems; ++k) {
-        float g = widen<DT>(graw, k);
+    for (int k = 0; k < EPL; ++k) {
+        float g = widen<DT, EPL>(graw, k);
         float pk = p[k];
         if constexpr (KIND == KIND_PLAIN) {
-            if (h.apply_decay && !h.decoupled) g = g + pk * h.wd;                // ref:1452-1453
-            if (h.apply_decay && h.decoupled) pk = pk * h.one_m_wd;              // ref:1454-1455
-            pk = pk - g * h.lr;                                                  // ref:1456
+            if (h.apply_decay && !h.decoupled) g = g + pk * h.wd;                   // ref:1452-1453
+            if (h.apply_decay && h.decoupled) pk = pk * h.one_m_wd;                 // ref:1454-1455
+            pk = pk - g * h.lr;                                                     // ref:1456
         } else {
-            if (KIND == KIND_SGD && !h.decoupled) g = g + pk * h.wd;             // ref:1639-1640
+            if (KIND == KIND_SGD && !h.decoupled) g = g + pk * h.wd;                // ref:1639-1640
             float mo;
-            if constexpr (QUANT) mo = lut_lane[byte_of(mraw, k) * 32] * sm;      // ref:1648-1657
-            else mo = widen<DT>(mraw, k);                                        // ref:1660-1661
+            if constexpr (QUANT) mo = StepLut::lookup(lut_lane, byte_of<EPL>(mraw, k)) * sm;   // ref:1648-1657
+            else mo = widen<DT, EPL>(mraw, k);                                      // ref:1660-1661
             float mn;
             if constexpr (KIND == KIND_LION) {
-                const float u = (mo * h.update_coef) + (g * h.one_m_update_coef);     // ref:1667
-                const float sgn = (u > 0.0f) ? 1.0f : ((u < 0.0f) ? -1.0f : 0.0f);   // ref:1668
-                mn = (mo * h.mom_coef) + (g * h.one_m_mom_coef);                      // ref:1669
-                pk = pk * h.one_m_wd;                                                 // ref:1675
-                pk = pk - sgn * h.lr;                                                 // ref:1676
+                const float u = (mo * h.update_coef) + (g * h.one_m_update_coef);        // ref:1667
+                const float sgn = (u > 0.0f) ? 1.0f : ((u < 0.0f) ? -1.0f : 0.0f);      // ref:1668
+                mn = (mo * h.mom_coef) + (g * h.one_m_mom_coef);                         // ref:1669
+                pk = pk * h.one_m_wd;                                                    // ref:1675
+                pk = pk - sgn * h.lr;                                                    // ref:1676
             } else {
-                mn = mo * h.mom_coef + g * h.update_coef;                             // ref:1671
-                if (h.decoupled) pk = pk * h.one_m_wd;                                // ref:1678-1679
-                if (h.nesterov) pk = pk - (g + h.mom_coef * mn) * h.lr;               // ref:1680-1681
-                else pk = pk - mn * h.lr;                                             // ref:1682-1683
+                mn = mo * h.mom_coef + g * h.update_coef;                                // ref:1671
+                if (h.decoupled) pk = pk * h.one_m_wd;                                   // ref:1678-1679
+                if (h.nesterov) pk = pk - (g + h.mom_coef * mn) * h.lr;                  // ref:1680-1681
+                else pk = pk - mn * h.lr;                                                // ref:1682-1683
             }
             m[k] = mn;
             am = fmaxf(am, fabsf(mn));
@@ -72,28 +72,28 @@ __device__ __forceinline__ void momentum_lane(const TensorPtrs& t, int64_t first
         p[k] = pk;
     }
 
-    Pack<ECCB> eout;
-    write_master<DT, ECCB>(p, praw, eout);                                       // ref:1684-1694
-    store_lane<PB, FAST>(praw, t.param, first, n);
-    store_lane<ECCB, FAST>(eout, t.ecc, first, n);
+    Pack<ECCB, EPL> eout;
+    write_master<DT, ECCB, EPL>(p, praw, eout);                                     // ref:1684-1694
+    store_lane<PB, EPL, FAST>(praw, t.param, first, n);
+    store_lane<ECCB, EPL, FAST>(eout, t.ecc, first, n);
 
     if constexpr (KIND != KIND_PLAIN) {
         if constexpr (QUANT) {
-            am = fmaxf(fmaxf(am, pair_swap(am)), 1e-12f);                        // ref:1702-1703
-            quantize_mom(m, am, mraw);
-            store_lane<1, FAST>(mraw, t.mom, first, n);
-            if (live_group && (threadIdx.x & 1) == 0) t.mom_scales[group] = f32_to_f16_bits(am);  // ref:1713-1716
+            am = fmaxf(group_max<EPL>(am), 1e-12f);                                 // ref:1702-1703
+            quantize_mom<EPL>(m, am, mraw);
+            store_lane<1, EPL, FAST>(mraw, t.mom, first, n);
+            if (live_group && (threadIdx.x & (32 / EPL - 1)) == 0) t.mom_scales[group] = f32_to_f16_bits(am);  // ref:1713-1716
         } else {
-            narrow_all<DT>(m, mraw);                                             // ref:1717-1719
-            store_lane<SB, FAST>(mraw, t.mom, first, n);
+            narrow_all<DT, EPL>(m, mraw);                                           // ref:1717-1719
+            store_lane<SB, EPL, FAST>(mraw, t.mom, first, n);
         }
     }
 }
 
-
 template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumOp {
     using Hyper = MomentumHyper;
     static constexpr bool kNeedsLut = QUANT && KIND != KIND_PLAIN;
+    static constexpr int kEpl = DTypeInfo<DT>::epl;
     template <bool FAST>
     __device__ __forceinline__ static void lane(const TensorPtrs& t, int64_t first, const Hyper& h, const float* lut) {
         momentum_lane<DT, ECCB, QUANT, KIND, FAST>(t, first, h, lut);

@@ -2,11 +2,11 @@
 // requantisation helpers, the two grid shapes (single tensor by value / chunk table over many tensors) and
 // the host-side launch + dispatch templates.
 //
-// Work decomposition: a block of 256 threads (4 wavefronts) owns one tile of 4096 consecutive elements of one
-// tensor.  Each lane owns 16 consecutive elements, so every stream (param, grad, ECC, codes) moves with
-// 128-bit loads/stores and one 32-element quantisation group is exactly two neighbouring lanes: the group
-// absmax is 15 in-register maxes plus one DPP quad-permute, no LDS round trip.  LDS only holds the
-// bank-replicated table that turns a first-moment code byte into its dequantised value.
+// Work decomposition.  The unit of scheduling is a tile of 4096 consecutive elements of one tensor; a block
+// (FO_BLOCK_THREADS threads) walks the tiles of its chunk, each wavefront taking sub-tiles of 64 x EPL
+// elements (EPL = 8 for bf16/fp16, 4 for fp32; see fo_device.h for the access shape).  A quantisation group is
+// 32/EPL neighbouring lanes, so the group absmax is in-register maxes plus two or three DPP moves.  LDS only
+// holds the table that turns a first-moment code byte into its dequantised value.
 //
 // "ref:" cites /root/reference/flashoptim/optimizers.py.
 #pragma once
@@ -15,7 +15,18 @@
 #include "fo_host.h"
 #include "../../include/flashoptim_hip.h"
 
+#ifndef FO_BLOCK_THREADS
+#define FO_BLOCK_THREADS 512
+#endif
+#ifndef FO_LUT_REPL
+#define FO_LUT_REPL 32
+#endif
+
 namespace fo {
+
+constexpr int kBlockThreads = FO_BLOCK_THREADS;
+constexpr int kBlockWaves = kBlockThreads / 64;
+using StepLut = Lut<FO_LUT_REPL>;
 
 struct TensorPtrs {
     void* param;
@@ -36,112 +47,119 @@ __device__ __forceinline__ TensorPtrs load_desc(const fo_tensor_desc* d) {
     return t;
 }
 
-// 128-bit accesses need every streamed pointer 16-byte aligned (tiles start at multiples of 4096 elements).
+// Vector accesses need every streamed pointer 16-byte aligned (tiles start at multiples of 4096 elements).
 __device__ __forceinline__ bool all_aligned16(const TensorPtrs& t) {
     const uintptr_t bits = (uintptr_t)t.param | (uintptr_t)t.grad | (uintptr_t)t.ecc | (uintptr_t)t.mom | (uintptr_t)t.var;
     return (bits & 15u) == 0;
 }
 
 // ------------------------------------------------------------------------------------------------
-// shared pieces of the two step kernels
+// shared pieces of the step kernels
 // ------------------------------------------------------------------------------------------------
 
-// Reads the 16 parameter values of the lane as fp32 masters (ref:2299-2309).
-template <int DT, int ECCB>
-__device__ __forceinline__ void read_master(float (&p)[kLaneElems], const Pack<DTypeInfo<DT>::bytes>& praw,
-                                            const Pack<ECCB>& eraw) {
+// Reads the lane's parameter values as fp32 masters (ref:2299-2309).
+template <int DT, int ECCB, int EPL>
+__device__ __forceinline__ void read_master(float (&p)[EPL], const Pack<DTypeInfo<DT>::bytes, EPL>& praw,
+                                            const Pack<ECCB, EPL>& eraw) {
 #pragma unroll
-    for (int k = 0; k < kLaneElems; ++k) {
-        const float w = widen<DT>(praw, k);
-        if constexpr (ECCB > 0) p[k] = ecc_join<DT, ECCB>(w, ecc_to_float<ECCB>(eraw, k));
+    for (int k = 0; k < EPL; ++k) {
+        const float w = widen<DT, EPL>(praw, k);
+        if constexpr (ECCB > 0) p[k] = ecc_join<DT, ECCB>(w, ecc_to_float<ECCB, EPL>(eraw, k));
         else p[k] = w;
     }
 }
 
 // Narrows the updated masters and derives the new ECC (ref:2377-2387).
-template <int DT, int ECCB>
-__device__ __forceinline__ void write_master(const float (&p)[kLaneElems], Pack<DTypeInfo<DT>::bytes>& pout,
-                                             Pack<ECCB>& eout) {
-    u32 eb[kLaneElems];
+template <int DT, int ECCB, int EPL>
+__device__ __forceinline__ void write_master(const float (&p)[EPL], Pack<DTypeInfo<DT>::bytes, EPL>& pout,
+                                             Pack<ECCB, EPL>& eout) {
+    u32 eb[EPL];
 #pragma unroll
-    for (int k = 0; k < kLaneElems; k += 2) {
+    for (int k = 0; k < EPL; k += 2) {
         float wa, wb;
-        narrow_pair<DT>(pout, k, p[k], p[k + 1], wa, wb);
+        narrow_pair<DT, EPL>(pout, k, p[k], p[k + 1], wa, wb);
         if constexpr (ECCB > 0) {
-            eb[k] = ecc_split_bits<DT, ECCB>(p[k], wa);
-            eb[k + 1] = ecc_split_bits<DT, ECCB>(p[k + 1], wb);
+            eb[k] = ecc_split_bits<DT, ECCB, false>(p[k], wa);
+            eb[k + 1] = ecc_split_bits<DT, ECCB, false>(p[k + 1], wb);
         }
     }
-    if constexpr (ECCB == 1) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) eout.w[i] = pack_bytes4(eb[4 * i], eb[4 * i + 1], eb[4 * i + 2], eb[4 * i + 3]);
-    }
-    if constexpr (ECCB == 2) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) eout.w[i] = pack_halves2(eb[2 * i], eb[2 * i + 1]);
-    }
+    if constexpr (ECCB > 0) pack_codes<ECCB, EPL>(eb, eout);
 }
 
-// Quantises the lane's 16 first-moment values against the group absmax `am` (already shared by the lane
-// pair, clamped at 1e-12): code = rne(127 * 2x/(1+|x|)), x = m/am  ==  rne(254 * m / (am + |m|))
+// Quantises the lane's first-moment values against the group absmax `am` (shared by the group's lanes,
+// clamped at 1e-12): code = rne(127 * 2x/(1+|x|)), x = m/am  ==  rne(254 * m / (am + |m|))
 // (ref:2407-2418 with the two divisions merged algebraically; one hardware reciprocal per element).
-__device__ __forceinline__ void quantize_mom(const float (&m)[kLaneElems], float am, Pack<1>& out) {
-    u32 b[kLaneElems];
+template <int EPL>
+__device__ __forceinline__ void quantize_mom(const float (&m)[EPL], float am, Pack<1, EPL>& out) {
+    u32 b[EPL];
 #pragma unroll
-    for (int k = 0; k < kLaneElems; ++k) {
+    for (int k = 0; k < EPL; ++k) {
         const float t = m[k] * __builtin_amdgcn_rcpf(am + fabsf(m[k]));
         b[k] = as_u32(fmaf(t, 254.0f, kMagic));
     }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) out.w[i] = pack_bytes4(b[4 * i], b[4 * i + 1], b[4 * i + 2], b[4 * i + 3]);
+    pack_codes<1, EPL>(b, out);
 }
 
 // Quantises sqrt(v): code = rne(255 * r / av) with 255/av formed once per lane (ref:2408-2419).
-__device__ __forceinline__ void quantize_var(const float (&r)[kLaneElems], float av, Pack<1>& out) {
+template <int EPL>
+__device__ __forceinline__ void quantize_var(const float (&r)[EPL], float av, Pack<1, EPL>& out) {
     const float scale = div_rn(255.0f, av);
-    u32 b[kLaneElems];
+    u32 b[EPL];
 #pragma unroll
-    for (int k = 0; k < kLaneElems; ++k) b[k] = as_u32(fmaf(r[k], scale, kMagic));
-#pragma unroll
-    for (int i = 0; i < 4; ++i) out.w[i] = pack_bytes4(b[4 * i], b[4 * i + 1], b[4 * i + 2], b[4 * i + 3]);
+    for (int k = 0; k < EPL; ++k) b[k] = as_u32(fmaf(r[k], scale, kMagic));
+    pack_codes<1, EPL>(b, out);
 }
 
-template <int DT>
-__device__ __forceinline__ void narrow_all(const float (&x)[kLaneElems], Pack<DTypeInfo<DT>::bytes>& out) {
+template <int DT, int EPL>
+__device__ __forceinline__ void narrow_all(const float (&x)[EPL], Pack<DTypeInfo<DT>::bytes, EPL>& out) {
 #pragma unroll
-    for (int k = 0; k < kLaneElems; k += 2) {
+    for (int k = 0; k < EPL; k += 2) {
         float wa, wb;
-        narrow_pair<DT>(out, k, x[k], x[k + 1], wa, wb);
+        narrow_pair<DT, EPL>(out, k, x[k], x[k + 1], wa, wb);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// kernels
+// ------------------------------------------------------------------------------------------------
+
+// One tile: every wavefront of the block takes sub-tiles wave, wave + W, ... of the tile.
+template <class Op>
+__device__ __forceinline__ void run_tile(const TensorPtrs& t, int64_t tile, bool aligned, const typename Op::Hyper& h,
+                                         const float* lut_lane) {
+    constexpr int kSub = 64 * Op::kEpl;              // elements per sub-tile
+    constexpr int kSubsPerTile = kTileElems / kSub;  // 8 (EPL 8) or 16 (EPL 4)
+    const int64_t tile_base = tile * (int64_t)kTileElems;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // block-uniform choice: whole tile in range and every stream 16-byte aligned -> straight-line vector path
+    if (aligned && (tile_base + kTileElems <= t.n)) {
+        for (int s = wave; s < kSubsPerTile; s += kBlockWaves)
+            Op::template lane<true>(t, tile_base + s * kSub + lane * Op::kEpl, h, lut_lane);
+    } else {
+        for (int s = wave; s < kSubsPerTile; s += kBlockWaves)
+            Op::template lane<false>(t, tile_base + s * kSub + lane * Op::kEpl, h, lut_lane);
     }
 }
 
 template <class Op>
-__device__ __forceinline__ void run_tile(const TensorPtrs& t, int64_t tile, bool aligned, const typename Op::Hyper& h,
-                                         const float* lut_lane) {
-    const int64_t tile_base = tile * (int64_t)kTileElems;
-    const int64_t first = tile_base + (int64_t)threadIdx.x * kLaneElems;
-    // block-uniform choice: whole tile in range and every stream 16-byte aligned -> straight-line 128-bit path
-    if (aligned && (tile_base + kTileElems <= t.n)) Op::template lane<true>(t, first, h, lut_lane);
-    else Op::template lane<false>(t, first, h, lut_lane);
-}
-
-template <class Op>
-__global__ __launch_bounds__(kBlockThreads) void step_single_kernel(TensorPtrs t, typename Op::Hyper h) {
-    __shared__ float lut[Op::kNeedsLut ? kLutFloats : 32];
-    if constexpr (Op::kNeedsLut) build_softsign_lut(lut);
-    const float* lut_lane = lut + (threadIdx.x & 31);
+__global__ __launch_bounds__(kBlockThreads) void step_single_kernel(TensorPtrs t, typename Op::Hyper h, int tiles_per_block) {
+    __shared__ float lut[Op::kNeedsLut ? StepLut::kFloats : 1];
+    if constexpr (Op::kNeedsLut) StepLut::build(lut);
+    const float* lut_lane = StepLut::lane_base(lut);
     const bool aligned = all_aligned16(t);
     const int64_t n_tiles = (t.n + kTileElems - 1) / kTileElems;
-    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) run_tile<Op>(t, tile, aligned, h, lut_lane);
+    const int64_t t0 = (int64_t)blockIdx.x * tiles_per_block;
+    const int64_t t1 = t0 + tiles_per_block < n_tiles ? t0 + tiles_per_block : n_tiles;
+    for (int64_t tile = t0; tile < t1; ++tile) run_tile<Op>(t, tile, aligned, h, lut_lane);
 }
 
 template <class Op>
 __global__ __launch_bounds__(kBlockThreads) void step_multi_kernel(const fo_tensor_desc* __restrict__ descs,
                                                                    const fo_chunk* __restrict__ chunks, int64_t n_chunks,
                                                                    typename Op::Hyper h) {
-    __shared__ float lut[Op::kNeedsLut ? kLutFloats : 32];
-    if constexpr (Op::kNeedsLut) build_softsign_lut(lut);
-    const float* lut_lane = lut + (threadIdx.x & 31);
+    __shared__ float lut[Op::kNeedsLut ? StepLut::kFloats : 1];
+    if constexpr (Op::kNeedsLut) StepLut::build(lut);
+    const float* lut_lane = StepLut::lane_base(lut);
     for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
         const fo_chunk ck = chunks[c];
         const TensorPtrs t = load_desc(descs + ck.tensor);
@@ -197,22 +215,20 @@ inline int validate_multi(const fo_tensor_desc* descs, int64_t n_tensors, const 
 
 template <class Op>
 int launch_single(const fo::TensorPtrs& t, const typename Op::Hyper& h, hipStream_t stream) {
+    // One pass over the tensor with many short-lived blocks: the hardware scheduler keeps neighbouring tiles
+    // in flight together, which streams from HBM measurably better than a persistent grid-stride loop.
     const int64_t n_tiles = (t.n + fo::kTileElems - 1) / fo::kTileElems;
-    const int cus = compute_units();
-    if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
-    const int64_t cap = (int64_t)cus * kBlocksPerCu;
-    const unsigned grid = (unsigned)(n_tiles < cap ? n_tiles : cap);
-    hipLaunchKernelGGL(fo::step_single_kernel<Op>, dim3(grid), dim3(fo::kBlockThreads), 0, stream, t, h);
+    const int tpb = tiles_per_block();
+    const int64_t grid = (n_tiles + tpb - 1) / tpb;
+    if (grid > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "tensor too large for one launch");
+    hipLaunchKernelGGL(fo::step_single_kernel<Op>, dim3((unsigned)grid), dim3(fo::kBlockThreads), 0, stream, t, h, tpb);
     return check_hip(hipGetLastError(), "step kernel launch");
 }
 
 template <class Op>
 int launch_multi(const fo_tensor_desc* descs, const fo_chunk* chunks, int64_t n_chunks, const typename Op::Hyper& h, hipStream_t stream) {
-    const int cus = compute_units();
-    if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
-    const int64_t cap = (int64_t)cus * kBlocksPerCu;
-    const unsigned grid = (unsigned)(n_chunks < cap ? n_chunks : cap);
-    hipLaunchKernelGGL(fo::step_multi_kernel<Op>, dim3(grid), dim3(fo::kBlockThreads), 0, stream, descs, chunks, n_chunks, h);
+    const int64_t grid = n_chunks < INT32_MAX ? n_chunks : INT32_MAX;  // one chunk per block; the loop covers the rest
+    hipLaunchKernelGGL(fo::step_multi_kernel<Op>, dim3((unsigned)grid), dim3(fo::kBlockThreads), 0, stream, descs, chunks, n_chunks, h);
     return check_hip(hipGetLastError(), "multi-tensor step kernel launch");
 }
 

@@ -299,6 +299,7 @@ def adam_step_ref(
         g = g + p * wd  # ref:2310-2311
     m = _load_state(mom, signed=True, sqrt=False, softsign=True)  # ref:2325-2343
     v = _load_state(var, signed=False, sqrt=True, softsign=False)  # ref:2326-2348
+    m_terms = (m * b1).abs() + (g * one_m_b1).abs()  # magnitude of what is summed into m (for error scales)
     m = m * b1 + g * one_m_b1  # ref:2357
     v = v * b2 + (g * g) * one_m_b2  # ref:2360
     if decoupled:
@@ -310,7 +311,9 @@ def adam_step_ref(
     _write_master(param.reshape(-1), None if ecc is None else ecc.reshape(-1), p)
     _store_state(mom, m, signed=True, sqrt=False, softsign=True)  # ref:2390-2434
     _store_state(var, v, signed=False, sqrt=True, softsign=False)
-    return {"p_before": p_before, "p_after": p, "m": m, "v": v}
+    # update_scale: size of the update with the terms of m taken in magnitude, i.e. what a relative rounding
+    # error of the update arithmetic scales with even when those terms cancel
+    return {"p_before": p_before, "p_after": p, "m": m, "v": v, "update_scale": (lr * (m_terms / bc1)) / denom}
 
 
 def momentum_step_ref(
@@ -349,11 +352,12 @@ def momentum_step_ref(
             p = p * one_m_wd
         p = p - g * lr
         _write_master(param.reshape(-1), eccf, p)
-        return {"p_before": p_before, "p_after": p}
+        return {"p_before": p_before, "p_after": p, "update_scale": (g * lr).abs()}
 
     if not do_lion and not decoupled:
         g = g + p * wd  # ref:1639-1640
     m = _load_state(mom, signed=True, sqrt=False, softsign=True)  # ref:1643-1661
+    m_terms = (m * mc).abs() + g.abs()
     if do_lion:
         one_m_uc = f32(np.float32(1.0) - np.float32(uc))
         one_m_mc = f32(np.float32(1.0) - np.float32(mc))
@@ -372,4 +376,5 @@ def momentum_step_ref(
             p = p - m * lr  # ref:1682-1683
     _write_master(param.reshape(-1), eccf, p)  # ref:1684-1694
     _store_state(mom, m, signed=True, sqrt=False, softsign=True)  # ref:1697-1719
-    return {"p_before": p_before, "p_after": p, "m": m}
+    scale = torch.full_like(p, lr) if do_lion else (m_terms + g.abs()) * lr
+    return {"p_before": p_before, "p_after": p, "m": m, "update_scale": scale}

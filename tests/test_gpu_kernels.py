@@ -159,7 +159,7 @@ class _Case:
     def compare(self, what, info):
         """`info`: the oracle's intermediates of the step just taken."""
         parity.check_master(self.gp, self.gecc, self.p, self.ecc, what,
-                            step_size=(info["p_after"] - info["p_before"]).abs())
+                            step_size=info["update_scale"])
         stats = []
         for i, (s, (a, b)) in enumerate(zip(self.states, self.gstates)):
             if self.quantized:
