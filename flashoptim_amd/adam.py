@@ -1,0 +1,122 @@
+"""FlashAdam / FlashAdamW (interface of ``/root/reference/flashoptim/optimizers.py:1784-2032``, cited ``ref:``)."""
+
+from __future__ import annotations
+
+from collections.abc import Iterable
+from typing import Any, Literal, Optional
+
+import torch
+
+from .base import FlashOptimizer, LaunchKey
+from .launcher import StepTensors
+from .state import QuantizedTensorSpec
+
+
+class FlashAdam(FlashOptimizer):
+    """Adam with L2 regularisation folded into the gradient, like ``torch.optim.Adam``.
+
+    Args:
+        params: parameters or param-group dicts.
+        lr: learning rate (default 1e-3).
+        betas: decay rates of the first and second moment (default (0.9, 0.999)).
+        eps: added to the denominator (default 1e-8).
+        weight_decay: L2 coefficient (default 0).
+        quantize, compress_state_dict, master_weight_bits, check_numerics, fused: see :class:`FlashOptimizer`.
+    """
+
+    def __init__(
+        self,
+        params: Iterable[torch.Tensor],
+        lr: float = 1e-3,
+        betas: tuple[float, float] = (0.9, 0.999),
+        eps: float = 1e-8,
+        weight_decay: float = 0.0,
+        quantize: bool = True,
+        compress_state_dict: bool = False,
+        master_weight_bits: Literal[24, 32] | None = 24,
+        check_numerics: bool = False,
+        fused: bool = True,
+    ):
+        if not 0.0 <= eps:
+            raise ValueError(f"Invalid epsilon value: {eps}")
+        for i, beta in enumerate(betas[:2]):
+            if not 0.0 <= beta <= 1.0:
+                raise ValueError(f"Invalid beta parameter at index {i}: {beta}")
+        if not 0.0 <= weight_decay:
+            raise ValueError(f"Invalid weight_decay value: {weight_decay}")
+        self._decoupled = False
+        self._decouple_lr = False
+        super().__init__(
+            params=params, lr=lr, defaults={"betas": betas, "weight_decay": weight_decay, "eps": eps},
+            quantize=quantize, compress_state_dict=compress_state_dict, master_weight_bits=master_weight_bits,
+            check_numerics=check_numerics, fused=fused,
+        )
+
+    def _quantized_state_spec(self) -> dict[str, QuantizedTensorSpec]:
+        return {
+            "exp_avg": QuantizedTensorSpec(signed=True, softsign=True),                    # int8, softsign
+            "exp_avg_sq": QuantizedTensorSpec(signed=False, sqrt=True, softsign=False),    # uint8 of sqrt(v)
+        }
+
+    def _ensure_state_initialized(self, p: torch.Tensor, hparams: dict[str, Any]) -> None:
+        super()._ensure_state_initialized(p, hparams)
+        state = self.state[p]
+        if "step" not in state:
+            # a CPU fp32 scalar like torch's own optimizers checkpoint it; reading it never syncs the device
+            state["step"] = torch.tensor(0, dtype=torch.float32, device="cpu")
+
+    def _min_step_size_relative_to_lr(self) -> float:
+        # |m| / sqrt(v) has no positive lower bound; assume updates routinely shrink to a tenth of lr
+        return 0.1
+
+    def _plan_step(self, param, grad, errors, param_state, hparams) -> Optional[tuple[LaunchKey, StepTensors]]:
+        lr = hparams["lr"]
+        weight_decay = hparams["weight_decay"]
+        if self._decoupled:  # the kernel multiplies the weights by 1 - weight_decay (ref:1894-1898)
+            weight_decay *= (lr / hparams["initial_lr"]) if self._decouple_lr else lr
+        exp_avg, exp_avg_sq = param_state["exp_avg"], param_state["exp_avg_sq"]
+        param_state["step"] += 1
+        scalars = (
+            ("lr", lr), ("beta1", hparams["betas"][0]), ("beta2", hparams["betas"][1]), ("eps", hparams["eps"]),
+            ("weight_decay", weight_decay), ("decoupled", self._decoupled), ("step", int(param_state["step"].item())),
+        )
+        key = LaunchKey("adam", param.dtype, 0 if errors is None else errors.element_size(), exp_avg.is_quantized(), scalars)
+        tensors = StepTensors(
+            param=param, grad=grad, ecc=errors,
+            mom=exp_avg.kernel_tensor, mom_scales=exp_avg.kernel_scales_or_self,
+            var=exp_avg_sq.kernel_tensor, var_scales=exp_avg_sq.kernel_scales_or_self,
+        )
+        return key, tensors
+
+
+class FlashAdamW(FlashAdam):
+    """AdamW: the decay multiplies the weights by ``1 - weight_decay * lr`` (``lr / initial_lr`` with
+    ``decouple_lr=True``) instead of entering the gradient.
+
+    Args:
+        weight_decay: decoupled decay coefficient (default 1e-2).
+        decouple_lr: scale the decay by ``lr / initial_lr`` instead of ``lr`` (default False).
+        Other arguments as :class:`FlashAdam`.
+    """
+
+    def __init__(
+        self,
+        params: Iterable[torch.Tensor],
+        lr: float = 1e-3,
+        betas: tuple[float, float] = (0.9, 0.999),
+        eps: float = 1e-8,
+        weight_decay: float = 1e-2,
+        decouple_lr: bool = False,
+        quantize: bool = True,
+        compress_state_dict: bool = False,
+        master_weight_bits: Optional[Literal[24, 32]] = 24,
+        check_numerics: bool = False,
+        fused: bool = True,
+    ):
+        super().__init__(
+            params, lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, quantize=quantize,
+            compress_state_dict=compress_state_dict, master_weight_bits=master_weight_bits,
+            check_numerics=check_numerics, fused=fused,
+        )
+        self._decoupled = True
+        self._decouple_lr = decouple_lr

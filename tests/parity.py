@@ -138,4 +138,6 @@ def check_master(param_gpu, ecc_gpu, param_ref, ecc_ref, what: str, step_size=No
 
 
 def bits_equal(a: torch.Tensor, b: torch.Tensor) -> bool:
-    return torch.equal(a.cpu().contiguous().view(torch.uint8), b.cpu().contiguous().view(torch.uint8))
+    if a.dtype != b.dtype or a.shape != b.shape:
+        return False
+    return torch.equal(a.cpu().contiguous().reshape(-1).view(torch.uint8), b.cpu().contiguous().reshape(-1).view(torch.uint8))
