@@ -1,0 +1,279 @@
+#!/usr/bin/env python3
+"""Throughput of the fused optimizer step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+A "step" is one pass of the optimizer over a resident synthetic parameter set (``optimizer.step()``: host
+planning plus the multi-tensor HIP launch).  W untimed warm-up steps, then exactly K steps between two
+``torch.cuda.synchronize()`` calls; one JSON line on stdout.
+
+Workloads (``--workload``):
+  llama8b-mwb24   default.  Llama-3-8B-shaped parameter list (291 tensors, 8 030 261 248 bf16 parameters),
+                  FlashAdamW, master_weight_bits=24, one multi-tensor launch per step: the configuration the
+                  headline metric is quoted on.
+  llama8b-mwb32   same shapes, master_weight_bits=32 (int16 correction term).
+  flat-2p30       one flat bf16 tensor of 2^30 elements, FlashAdamW, master_weight_bits=24.
+  ragged-lion / ragged-sgdw
+                  4096 bf16 tensors with log-uniform lengths in [1, 2^24] (~1e9 parameters), FlashLion / FlashSGDW.
+  llama8b-fp32-release
+                  fp32 parameters, quantised moments, one launch per tensor in reverse order as under gradient
+                  release; ends with a compressed state_dict save -> load round trip checked bit for bit.
+
+Reported: ``value`` = parameters updated per second; ``roofline`` = algorithmic HBM bytes of one step divided
+by the average duration of a step measured with events on the launch stream, against the 8 TB/s peak;
+``cpu_baseline`` = the CPU oracle (oracle/torch_oracle.py, all host cores) on a bounded sample of the same
+distribution, a reported baseline only.
+"""
+
+from __future__ import annotations
+
+import argparse
+import io
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+
+
+def llama3_8b_shapes():
+    """(name, shape) of the 291 tensors of a Llama-3-8B: 32 layers, hidden 4096, FFN 14336, 32 query / 8 KV heads of
+    128, vocabulary 128256 with untied embedding and lm_head, RMSNorm weights of length 4096."""
+    h, ffn, kv, vocab = 4096, 14336, 1024, 128256
+    shapes = [("embed", (vocab, h))]
+    for i in range(32):
+        shapes += [(f"l{i}.q", (h, h)), (f"l{i}.k", (kv, h)), (f"l{i}.v", (kv, h)), (f"l{i}.o", (h, h)),
+                   (f"l{i}.gate", (ffn, h)), (f"l{i}.up", (ffn, h)), (f"l{i}.down", (h, ffn)),
+                   (f"l{i}.ln1", (h,)), (f"l{i}.ln2", (h,))]
+    shapes += [("norm", (h,)), ("lm_head", (vocab, h))]
+    return shapes
+
+
+def ragged_lengths(count=4096, total=1_000_000_000, seed=3):
+    """Lengths floor(2^(24 U)) clipped to [1, 2^24], rescaled towards `total`, with the lengths 1, 31, 33 present
+    and at least a quarter of them not multiples of the group size."""
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.floor(torch.exp2(24.0 * torch.rand(count, generator=g, dtype=torch.float64))).clamp(1, 1 << 24)
+    lens = torch.floor(lens * (total / lens.sum().item())).clamp(1, 1 << 24).to(torch.int64)
+    lens[:3] = torch.tensor([1, 31, 33])
+    odd = lens % 32 == 0
+    fix = torch.nonzero(odd).flatten()[: max(0, count // 4 - int((~odd).sum()))]
+    lens[fix] += 1
+    return lens.tolist()
+
+
+def bytes_per_param(param_bytes: int, ecc_bytes: int, n_states: int) -> float:
+    """Algorithmic HBM traffic of one element: read param, grad, ecc, codes, scales; write all but grad."""
+    state = n_states * (1.0 + 2.0 / 32.0)
+    return (2 * param_bytes + ecc_bytes + state) + (param_bytes + ecc_bytes + state)
+
+
+def make_params(shapes, dtype, device, grad_scales=None, seed=0):
+    torch.manual_seed(seed)
+    params = []
+    for i, (name, shape) in enumerate(shapes):
+        if len(shape) == 1 and ("ln" in name or name == "norm"):
+            w = torch.ones(shape, device=device, dtype=dtype)
+        else:
+            w = (torch.randn(shape, device=device, dtype=torch.float32) * 0.02).to(dtype)
+        p = torch.nn.Parameter(w)
+        s = 1.0 if grad_scales is None else grad_scales[i]
+        p.grad = (torch.randn(shape, device=device, dtype=torch.float32) * (1e-3 * s)).to(dtype)
+        params.append(p)
+    return params
+
+
+def build_workload(name: str, device):
+    import flashoptim_amd as fo
+
+    hp = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+    if name in ("llama8b-mwb24", "llama8b-mwb32"):
+        shapes = llama3_8b_shapes()
+        g = torch.Generator().manual_seed(2)
+        scales = (10.0 ** (torch.rand(len(shapes), generator=g) * 2 - 1)).tolist()
+        params = make_params(shapes, torch.bfloat16, device, scales)
+        mwb = 24 if name.endswith("24") else 32
+        opt = fo.FlashAdamW(params, master_weight_bits=mwb, **hp)
+        return dict(params=params, opt=opt, step=opt.step, bpp=bytes_per_param(2, 1 if mwb == 24 else 2, 2),
+                    desc=f"Llama-3-8B-shaped parameter list, bf16, FlashAdamW, master_weight_bits={mwb}",
+                    launch="one multi-tensor launch per step", optimizer="FlashAdamW", mwb=mwb)
+    if name == "flat-2p30":
+        params = make_params([("flat", (1 << 30,))], torch.bfloat16, device)
+        opt = fo.FlashAdamW(params, master_weight_bits=24, **hp)
+        return dict(params=params, opt=opt, step=opt.step, bpp=bytes_per_param(2, 1, 2),
+                    desc="one flat bf16 tensor of 2^30 elements, FlashAdamW, master_weight_bits=24",
+                    launch="one single-tensor launch per step", optimizer="FlashAdamW", mwb=24)
+    if name in ("ragged-lion", "ragged-sgdw"):
+        lens = ragged_lengths()
+        torch.manual_seed(3)
+        params = []
+        student = torch.distributions.StudentT(torch.tensor(3.0, device=device))
+        for n in lens:
+            p = torch.nn.Parameter((torch.randn(n, device=device) * 0.02).to(torch.bfloat16))
+            p.grad = (student.sample((n,)) * 1e-3).to(torch.bfloat16)
+            params.append(p)
+        if name == "ragged-lion":
+            opt = fo.FlashLion(params, lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1, master_weight_bits=24)
+        else:
+            opt = fo.FlashSGDW(params, momentum=0.9, lr=1e-2, weight_decay=1e-4, master_weight_bits=24)
+        return dict(params=params, opt=opt, step=opt.step, bpp=bytes_per_param(2, 1, 1),
+                    desc="4096 bf16 tensors, lengths log-uniform in [1, 2^24], Student-t(3) gradients, "
+                         + type(opt).__name__ + ", master_weight_bits=24",
+                    launch="one multi-tensor launch per step", optimizer=type(opt).__name__, mwb=24)
+    if name == "llama8b-fp32-release":
+        shapes = llama3_8b_shapes()
+        g = torch.Generator().manual_seed(2)
+        scales = (10.0 ** (torch.rand(len(shapes), generator=g) * 2 - 1)).tolist()
+        params = make_params(shapes, torch.float32, device, scales)
+        opt = fo.FlashAdamW(params, master_weight_bits=None, compress_state_dict=True, **hp)
+        group = opt.param_groups[0]
+
+        def step():  # what the gradient-release hooks do, in the order backward produces gradients
+            for p in reversed(params):
+                opt.step_param(p, group)
+
+        return dict(params=params, opt=opt, step=step, bpp=bytes_per_param(4, 0, 2),
+                    desc="Llama-3-8B-shaped parameter list, fp32 parameters, FlashAdamW, quantised moments, stepped "
+                         "per tensor in reverse order as under gradient release",
+                    launch="one single-tensor launch per tensor (291 per step)", optimizer="FlashAdamW", mwb=None,
+                    checkpoint_roundtrip=True)
+    raise SystemExit(f"unknown workload {name!r}")
+
+
+def checkpoint_roundtrip(work, device) -> bool:
+    """Compressed state_dict -> torch.save -> torch.load -> load_state_dict into a fresh optimizer; codes, fp16
+    scales and step counters must come back bit for bit (fp32 parameters)."""
+    import flashoptim_amd as fo
+
+    opt = work["opt"]
+    buf = io.BytesIO()
+    torch.save(opt.state_dict(), buf)
+    size = buf.tell()
+    buf.seek(0)
+    loaded = torch.load(buf, weights_only=True)
+    fresh = fo.FlashAdamW(work["params"], master_weight_bits=None, compress_state_dict=True, lr=1e-3)
+    fresh.load_state_dict(loaded)
+    ok = True
+    for p in work["params"]:
+        a, b = opt.state[p], fresh.state[p]
+        for k in ("exp_avg", "exp_avg_sq"):
+            ok &= torch.equal(a[k].quantized, b[k].quantized)
+            ok &= torch.equal(a[k].scales.view(torch.int16), b[k].scales.view(torch.int16))
+        ok &= a["step"].item() == b["step"].item()
+    work["checkpoint_bytes"] = size
+    return bool(ok)
+
+
+def cpu_baseline(steps: int = 5, warmup: int = 3, n: int = 1 << 26):
+    """The CPU oracle on a bounded sample: one flat bf16 tensor of 2^26 elements drawn like the flat workload
+    (params N(0, 0.02) seed 0, gradients N(0, 1e-3) seed 1000 + step), FlashAdamW master_weight_bits=24."""
+    from oracle import torch_oracle as T
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    p = (torch.randn(n, generator=torch.Generator().manual_seed(0)) * 0.02).to(torch.bfloat16)
+    ecc = torch.zeros(n, dtype=torch.int8)
+    m, v = T.MomentState.zeros(n, True, True, torch.bfloat16), T.MomentState.zeros(n, False, True, torch.bfloat16)
+    elapsed = 0.0
+    for step in range(1, warmup + steps + 1):
+        g = (torch.randn(n, generator=torch.Generator().manual_seed(1000 + step)) * 1e-3).to(torch.bfloat16)
+        t0 = time.perf_counter()
+        T.adam_step_ref(m, v, p, g, ecc, 1e-3, 0.9, 0.999, 1e-8, 0.01 * 1e-3, True, step)
+        if step > warmup:
+            elapsed += time.perf_counter() - t0
+    return {
+        "value": n * steps / elapsed, "unit": "params/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"FlashAdamW mwb=24 on one flat bf16 tensor of 2^26 elements, {warmup} warm-up + {steps} timed steps "
+                  "of the PyTorch CPU restatement (oracle/torch_oracle.py)",
+    }
+
+
+def measured_traffic(workload: str):
+    """HBM bytes per step measured with rocprofv3 FETCH_SIZE / WRITE_SIZE (see profiles/), if recorded."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(workload, {}).get("bytes_per_step")
+    except (OSError, ValueError):
+        return None
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="llama8b-mwb24")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: the optimizer step is shard-local and this build has no "
+                         "multi-GPU path (run with --gpus 1).")
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a ROCm GPU")
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    work = build_workload(args.workload, device)
+    step = work["step"]
+    total = sum(p.numel() for p in work["params"])
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for a, b in events:
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    device_ms = sorted(a.elapsed_time(b) for a, b in events)
+    avg_device_ms = sum(device_ms) / len(device_ms)
+
+    step_bytes = total * work["bpp"]
+    achieved = step_bytes / (avg_device_ms * 1e-3) / 1e9
+    out = {
+        "metric": "params updated/sec + achieved HBM GB/s (% peak), FlashAdamW step on 8B params",
+        "value": total / (ms_per_step * 1e-3),
+        "unit": "params/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": args.workload, "description": work["desc"], "optimizer": work["optimizer"],
+            "master_weight_bits": work["mwb"], "n_tensors": len(work["params"]), "n_params": total,
+            "launch": work["launch"], "algorithmic_bytes_per_param": work["bpp"],
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(args.workload),
+            "step_device_ms_avg": avg_device_ms, "step_device_ms_median": device_ms[len(device_ms) // 2],
+            "step_device_ms_min": device_ms[0], "algorithmic_bytes_per_step": step_bytes,
+        },
+    }
+    if work.get("checkpoint_roundtrip"):
+        out["config"]["checkpoint_roundtrip_bit_exact"] = checkpoint_roundtrip(work, device)
+        out["config"]["checkpoint_bytes"] = work["checkpoint_bytes"]
+    if not args.no_cpu_baseline:
+        del work
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
