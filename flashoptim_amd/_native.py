@@ -15,7 +15,10 @@ from typing import Optional
 import torch
 
 _LIB_NAME = "libflashoptim_hip.so"
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", _LIB_NAME)
+# FLASHOPTIM_HIP_LIBRARY points at an alternative build of the same library (kernel tuning); default: in-tree
+_LIB_PATH = os.environ.get("FLASHOPTIM_HIP_LIBRARY") or os.path.join(
+    os.path.dirname(os.path.abspath(__file__)), "lib", _LIB_NAME
+)
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 TILE_ELEMS = 4096

@@ -41,12 +41,19 @@ int check_hip(hipError_t e, const char* what) {
 
 const char* last_error() { return g_err; }
 
+static int env_int(const char* name, int fallback) {
+    const char* e = getenv(name);
+    const int v = e ? atoi(e) : 0;
+    return (v >= 1 && v <= 1024) ? v : fallback;
+}
+
 int tiles_per_block() {
-    static const int value = [] {
-        const char* e = getenv("FO_TILES_PER_BLOCK");
-        const int v = e ? atoi(e) : 0;
-        return (v >= 1 && v <= 1024) ? v : 4;
-    }();
+    static const int value = env_int("FO_TILES_PER_BLOCK", 1);
+    return value;
+}
+
+int default_tiles_per_chunk() {
+    static const int value = env_int("FO_TILES_PER_CHUNK", 1);
     return value;
 }
 
@@ -80,7 +87,7 @@ int fo_device_compute_units(int device) {
 
 int64_t fo_count_chunks(const int64_t* numels, int64_t n_tensors, int tiles_per_chunk) {
     if (!numels || n_tensors < 0) return fail(FO_ERR_INVALID_ARGUMENT, "bad tensor length array");
-    const int64_t tpc = tiles_per_chunk > 0 ? tiles_per_chunk : kDefaultTilesPerChunk;
+    const int64_t tpc = tiles_per_chunk > 0 ? tiles_per_chunk : default_tiles_per_chunk();
     int64_t total = 0;
     for (int64_t i = 0; i < n_tensors; ++i) {
         if (numels[i] < 0) return fail(FO_ERR_INVALID_ARGUMENT, "tensor %lld has negative length", (long long)i);
@@ -95,7 +102,7 @@ int64_t fo_build_chunks(const int64_t* numels, int64_t n_tensors, int tiles_per_
     if (need < 0) return need;
     if (!out || capacity < need) return fail(FO_ERR_INVALID_ARGUMENT, "chunk buffer too small (%lld < %lld)", (long long)capacity, (long long)need);
     if (n_tensors > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "too many tensors");
-    const int64_t tpc = tiles_per_chunk > 0 ? tiles_per_chunk : kDefaultTilesPerChunk;
+    const int64_t tpc = tiles_per_chunk > 0 ? tiles_per_chunk : default_tiles_per_chunk();
     int64_t c = 0;
     for (int64_t i = 0; i < n_tensors; ++i) {
         const int64_t tiles = (numels[i] + fo::kTileElems - 1) / fo::kTileElems;

@@ -20,7 +20,10 @@ const char* last_error();
 // FO_TILES_PER_BLOCK in the environment overrides it (read once; for tuning).
 int tiles_per_block();
 
+// Tiles per work item of the multi-tensor chunk table when the caller passes tiles_per_chunk <= 0.
+// FO_TILES_PER_CHUNK in the environment overrides it (read once; for tuning).
+int default_tiles_per_chunk();
+
 constexpr int kBlocksPerCu = 8;           // grid cap of the cold-path kernels: blocks per compute unit
-constexpr int kDefaultTilesPerChunk = 4;  // multi-tensor work item = 4 tiles = 16384 elements
 
 }  // namespace fo_host

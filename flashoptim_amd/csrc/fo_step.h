@@ -19,7 +19,7 @@
 #define FO_BLOCK_THREADS 512
 #endif
 #ifndef FO_LUT_REPL
-#define FO_LUT_REPL 32
+#define FO_LUT_REPL 1
 #endif
 
 namespace fo {
