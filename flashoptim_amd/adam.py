@@ -7,8 +7,7 @@ from typing import Any, Literal, Optional
 
 import torch
 
-from .base import FlashOptimizer, LaunchKey
-from .launcher import StepTensors
+from .base import FlashOptimizer
 from .state import QuantizedTensorSpec
 
 
@@ -69,24 +68,23 @@ class FlashAdam(FlashOptimizer):
         # |m| / sqrt(v) has no positive lower bound; assume updates routinely shrink to a tenth of lr
         return 0.1
 
-    def _plan_step(self, param, grad, errors, param_state, hparams) -> Optional[tuple[LaunchKey, StepTensors]]:
+    def _kernel_kind(self, hparams: dict[str, Any]) -> str:
+        return "adam"
+
+    def _moment_names(self, kind: str) -> tuple[Optional[str], Optional[str]]:
+        return "exp_avg", "exp_avg_sq"
+
+    def _advance_step(self, param_state: dict[str, Any]) -> Optional[int]:
+        param_state["step"] += 1
+        return int(param_state["step"].item())
+
+    def _kernel_scalars(self, hparams: dict[str, Any], step: Optional[int]) -> dict[str, Any]:
         lr = hparams["lr"]
         weight_decay = hparams["weight_decay"]
         if self._decoupled:  # the kernel multiplies the weights by 1 - weight_decay (ref:1894-1898)
             weight_decay *= (lr / hparams["initial_lr"]) if self._decouple_lr else lr
-        exp_avg, exp_avg_sq = param_state["exp_avg"], param_state["exp_avg_sq"]
-        param_state["step"] += 1
-        scalars = (
-            ("lr", lr), ("beta1", hparams["betas"][0]), ("beta2", hparams["betas"][1]), ("eps", hparams["eps"]),
-            ("weight_decay", weight_decay), ("decoupled", self._decoupled), ("step", int(param_state["step"].item())),
-        )
-        key = LaunchKey("adam", param.dtype, 0 if errors is None else errors.element_size(), exp_avg.is_quantized(), scalars)
-        tensors = StepTensors(
-            param=param, grad=grad, ecc=errors,
-            mom=exp_avg.kernel_tensor, mom_scales=exp_avg.kernel_scales_or_self,
-            var=exp_avg_sq.kernel_tensor, var_scales=exp_avg_sq.kernel_scales_or_self,
-        )
-        return key, tensors
+        return dict(lr=lr, beta1=hparams["betas"][0], beta2=hparams["betas"][1], eps=hparams["eps"],
+                    weight_decay=weight_decay, decoupled=self._decoupled, step=step)
 
 
 class FlashAdamW(FlashAdam):

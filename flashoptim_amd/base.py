@@ -2,10 +2,11 @@
 
 Same constructor arguments, param-group keys, per-parameter state layout, ``state_dict`` / ``load_state_dict``
 format and error behaviour as the reference base class (``/root/reference/flashoptim/optimizers.py:317-1203``,
-cited as ``ref:``).  What differs is underneath: subclasses describe a parameter's update as a *launch plan*
-(kernel kind, specialisation, fp32 scalars, raw tensors); ``step_param`` executes one plan with a single-tensor
-HIP launch, ``step`` groups the plans of all parameters into buckets and issues one multi-tensor launch per
-bucket.  There is no eager PyTorch implementation of the update in this package.
+cited as ``ref:``).  What differs is underneath: subclasses describe a param group's update as a kernel kind plus
+fp32 scalars; ``step_param`` executes one parameter with a single-tensor HIP launch, ``step`` groups the
+parameters into buckets and issues one multi-tensor launch per bucket, caching the per-parameter host work of a
+group whose parameter list and gradient layout did not change.  There is no eager PyTorch implementation of
+the update in this package.
 """
 
 from __future__ import annotations
@@ -23,7 +24,7 @@ import torch.nn as nn
 
 from . import kernels
 from .kernels import compute_ecc_bits, reconstruct_fp32_param
-from .launcher import MultiTensorLauncher, StepTensors
+from .launcher import BucketPlan, StepTensors
 from .state import QuantizedTensorSpec, _MaybeQuantizedTensor
 
 _DTYPE_WIDTHS = {torch.int8: 1, torch.int16: 2, torch.float16: 2, torch.bfloat16: 2, torch.float32: 4}
@@ -56,6 +57,29 @@ class LaunchKey:
     ecc_bytes: int
     quantized: bool
     scalars: tuple            # keyword arguments of the kernel wrapper, as a sorted tuple of items
+
+
+@dataclass
+class _Bucket:
+    """Cached launch state of the tensors of one param group that share a LaunchKey up to the scalars."""
+
+    kind: str
+    dtype: torch.dtype
+    ecc_bytes: int
+    quantized: bool
+    params: list                      # the nn.Parameters, in table order
+    tensors: list                     # StepTensors with grad=None (state tensors only)
+    plan: Optional[BucketPlan]        # multi-tensor tables; None for single-tensor / momentum-free buckets
+    step_tensors: list                # the CPU `step` scalars of the bucket (Adam), else empty
+    step_value: Optional[int]
+
+
+@dataclass
+class _GroupCache:
+    epoch: int
+    params: list
+    signature: Any
+    buckets: list
 
 
 class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
@@ -124,7 +148,8 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         self._check_numerics = check_numerics
         self._transient_state: dict[int, dict[str, Any]] = {}  # id(param) -> {"maxabs": ...}; never serialised
         self._gradient_release = False
-        self._launcher = MultiTensorLauncher()
+        self._plan_epoch = 0                       # bumped whenever cached launch plans may be stale
+        self._group_cache: dict[int, _GroupCache] = {}
 
         group_defaults = dict(defaults or {})
         group_defaults.update(lr=lr, initial_lr=lr, master_bytewidth=master_bytewidth, quantize=quantize)
@@ -165,16 +190,26 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         """Names and companding of the quantisable states, e.g. ``{"exp_avg": ..., "exp_avg_sq": ...}``."""
 
     @abc.abstractmethod
-    def _plan_step(
-        self,
-        param: torch.Tensor,
-        grad: torch.Tensor,
-        errors: Optional[torch.Tensor],
-        param_state: dict[str, Any],
-        hparams: dict[str, Any],
-    ) -> Optional[tuple[LaunchKey, StepTensors]]:
-        """Host-side part of one parameter's step: advance counters, fold the group's hyper-parameters into the
-        kernel scalars (in double, like the reference's ``_do_step``) and name the tensors.  ``None`` = no-op."""
+    def _kernel_kind(self, hparams: dict[str, Any]) -> str:
+        """"adam", "momentum" or "plain" (momentum-free SGD) for the tensors of this param group."""
+
+    @abc.abstractmethod
+    def _kernel_scalars(self, hparams: dict[str, Any], step: Optional[int]) -> dict[str, Any]:
+        """The kernel's scalar arguments for this param group, folded in double like the reference's ``_do_step``
+        (decoupled decay times lr, Lion's beta roles, ...)."""
+
+    @abc.abstractmethod
+    def _moment_names(self, kind: str) -> tuple[Optional[str], Optional[str]]:
+        """State keys of the first and second moment used by `kind` (None where there is none)."""
+
+    def _advance_step(self, param_state: dict[str, Any]) -> Optional[int]:
+        """Optimizers with bias correction advance and return their per-parameter step counter here."""
+        del param_state
+        return None
+
+    def _plan_signature(self, hparams: dict[str, Any]) -> Any:
+        """Whatever besides the parameter list decides which kernel a group uses; a change invalidates caches."""
+        return self._kernel_kind(hparams)
 
     def _initial_value_for_state_var(self, param: torch.Tensor, key: str) -> torch.Tensor:
         del key
@@ -223,7 +258,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
                 "recompute_param_stats() throughout training to fail faster and avoid this surprise."
             )
 
-    # ------------------------------------------------------------------------------------------- stepping
+    # --------------------------------------------------------------------------------- per-parameter plan
     def _ensure_state_initialized(self, p: torch.Tensor, hparams: dict[str, Any]) -> None:
         if self._check_numerics and self._transient_state.get(id(p), {}).get("maxabs") is None:
             self._recompute_stats_for_param(p)
@@ -246,6 +281,34 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
             if any(q is p for q in group["params"]):
                 return group
         raise ValueError(f"Parameter {p.shape} {p.dtype} not managed by this optimizer.")
+
+    def _plan_step(
+        self,
+        param: torch.Tensor,
+        grad: torch.Tensor,
+        errors: Optional[torch.Tensor],
+        param_state: dict[str, Any],
+        hparams: dict[str, Any],
+    ) -> tuple[LaunchKey, StepTensors]:
+        """Host-side part of one parameter's step: advance counters, fold the hyper-parameters into the kernel
+        scalars and name the tensors."""
+        if errors is not None and errors.dtype not in (torch.int8, torch.int16):
+            raise ValueError("Errors needs to be int8 or int16")
+        kind = self._kernel_kind(hparams)
+        scalars = self._kernel_scalars(hparams, self._advance_step(param_state))
+        mom_name, var_name = self._moment_names(kind)
+        mom = param_state[mom_name] if mom_name else None
+        var = param_state[var_name] if var_name else None
+        key = LaunchKey(kind, param.dtype, 0 if errors is None else errors.element_size(),
+                        mom.is_quantized() if mom is not None else False, tuple(sorted(scalars.items())))
+        tensors = StepTensors(
+            param=param, grad=grad, ecc=errors,
+            mom=None if mom is None else mom.kernel_tensor,
+            mom_scales=None if mom is None else mom.kernel_scales_or_self,
+            var=None if var is None else var.kernel_tensor,
+            var_scales=None if var is None else var.kernel_scales_or_self,
+        )
+        return key, tensors
 
     def _plan_param(self, p: torch.Tensor, group: dict[str, Any]) -> Optional[tuple[LaunchKey, StepTensors]]:
         """Everything ``step_param`` does short of launching (ref:699-759)."""
@@ -288,17 +351,6 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         else:
             kernels._sgd_plain_step(t.param, t.grad, t.ecc, **kw)
 
-    def _launch_bucket(self, key: LaunchKey, tensors: list[StepTensors]) -> None:
-        if len(tensors) == 1 or key.kind == "plain":
-            for t in tensors:
-                self._launch_single(key, t)
-            return
-        kw = dict(key.scalars)
-        if key.kind == "adam":
-            self._launcher.adam(tensors, key.dtype, key.ecc_bytes, key.quantized, **kw)
-        else:
-            self._launcher.momentum(tensors, key.dtype, key.ecc_bytes, key.quantized, **kw)
-
     @torch.no_grad()
     def step_param(self, p: torch.Tensor, group: Optional[dict[str, Any]] = None) -> None:
         """Step one parameter now (its ``.grad`` must be set).  Entry point of the gradient-release hooks.
@@ -309,9 +361,82 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         """
         if group is None:
             group = self._find_group(p)
+        self._plan_epoch += 1  # counters move outside step(): cached bucket state is stale
         plan = self._plan_param(p, group)
         if plan is not None:
             self._launch_single(*plan)
+
+    # -- step(): one multi-tensor launch per bucket, with the host work of an unchanged group cached ------------
+    def _step_group_slow(self, index: int, group: dict[str, Any]) -> None:
+        """Full per-parameter planning (state creation, checks, counters), then one launch per bucket; leaves a
+        cache behind when every parameter of the group took part."""
+        planned: dict[LaunchKey, list] = {}
+        complete = not self._check_numerics
+        for p in group["params"]:
+            plan = self._plan_param(p, group)
+            if plan is None:
+                complete = False
+                continue
+            key, tensors = plan
+            planned.setdefault(key, []).append((p, tensors))
+            if tensors.param is not p:
+                complete = False  # sharded wrapper: keep the generic path
+        buckets = []
+        for key, items in planned.items():
+            tensors = [t for _, t in items]
+            scalars = dict(key.scalars)
+            plan = None
+            if key.kind != "plain" and len(tensors) > 1:
+                plan = BucketPlan(key.kind, key.dtype, key.ecc_bytes, key.quantized, tensors)
+                plan.launch(**scalars)
+            else:
+                for t in tensors:
+                    self._launch_single(key, t)
+            step_tensors = [self.state[p]["step"] for p, _ in items] if "step" in scalars else []
+            for t in tensors:
+                t.grad = None  # the cache must not keep gradients alive
+            buckets.append(_Bucket(key.kind, key.dtype, key.ecc_bytes, key.quantized, [p for p, _ in items], tensors,
+                                   plan, step_tensors, scalars.get("step")))
+        if complete and buckets:
+            self._group_cache[index] = _GroupCache(self._plan_epoch, list(group["params"]),
+                                                   self._plan_signature(group), buckets)
+        else:
+            self._group_cache.pop(index, None)
+
+    def _step_group_fast(self, cache: _GroupCache, group: dict[str, Any]) -> bool:
+        """Re-issue the cached launches of a group whose parameters all have gradients of the cached layout.
+        Returns False (having changed nothing) when the group must go through the full path instead."""
+        moved = []
+        for b in cache.buckets:
+            ptrs = b.plan.grad_ptrs if b.plan is not None else None
+            for i, p in enumerate(b.params):
+                g = p.grad
+                if g is None or not p.requires_grad:
+                    return False
+                if ptrs is not None:
+                    ptr = g.data_ptr()
+                    if ptr != ptrs[i]:
+                        if g.dtype != b.dtype or g.device != p.device or not g.is_contiguous() or g.numel() != p.numel():
+                            return False
+                        moved.append((b.plan, i, ptr))
+                elif g.dtype != b.dtype or g.device != p.device or not g.is_contiguous():
+                    return False
+        for plan, i, ptr in moved:
+            plan.set_grad_ptr(i, ptr)
+        for b in cache.buckets:
+            if b.step_tensors:
+                torch._foreach_add_(b.step_tensors, 1)
+                b.step_value += 1
+            scalars = self._kernel_scalars(group, b.step_value)
+            if b.plan is not None:
+                b.plan.launch(**scalars)
+            else:
+                key = LaunchKey(b.kind, b.dtype, b.ecc_bytes, b.quantized, tuple(sorted(scalars.items())))
+                for p, t in zip(b.params, b.tensors):
+                    t.grad = p.grad
+                    self._launch_single(key, t)
+                    t.grad = None
+        return True
 
     @torch.no_grad()
     def step(self, closure: Optional[Callable] = None) -> Optional[torch.Tensor]:
@@ -326,15 +451,19 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         if closure is not None:
             with torch.enable_grad():
                 loss = closure()
-        buckets: dict[tuple, list[StepTensors]] = {}
-        for group in self.param_groups:
-            for p in group["params"]:
-                plan = self._plan_param(p, group)
-                if plan is not None:
-                    key, tensors = plan
-                    buckets.setdefault((key, tensors.param.device), []).append(tensors)
-        for (key, _device), tensors in buckets.items():
-            self._launch_bucket(key, tensors)
+        for index, group in enumerate(self.param_groups):
+            cache = self._group_cache.get(index)
+            if (
+                cache is not None
+                and cache.epoch == self._plan_epoch
+                and not self._check_numerics
+                and len(cache.params) == len(group["params"])
+                and all(a is b for a, b in zip(cache.params, group["params"]))
+                and cache.signature == self._plan_signature(group)
+                and self._step_group_fast(cache, group)
+            ):
+                continue
+            self._step_group_slow(index, group)
         return loss
 
     def zero_grad(self, set_to_none: bool = True) -> None:
@@ -346,6 +475,11 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
             )
             return
         super().zero_grad(set_to_none=set_to_none)
+
+    def add_param_group(self, param_group: dict[str, Any]) -> None:
+        super().add_param_group(param_group)
+        if hasattr(self, "_plan_epoch"):
+            self._plan_epoch += 1
 
     # ------------------------------------------------------------------------------------ (de)serialisation
     def _state_dict_for_param(self, param_number: int, opt_state: dict[int, Any], hparams: dict[str, Any],
@@ -435,8 +569,9 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
             # after the per-parameter pass, so that a master_bytewidth found there is known to come from the file
             group.setdefault("master_bytewidth", self._master_bytewidth)
         super().__setstate__(state)
-        if hasattr(self, "_launcher"):
-            self._launcher.clear()  # state tensors were replaced: cached pointer tables are stale
+        # state tensors were replaced: cached pointer tables and step counters are stale
+        self._plan_epoch = getattr(self, "_plan_epoch", 0) + 1
+        self._group_cache = {}
 
     def load_state_dict(self, state_dict: dict[str, Any]) -> None:
         """Also accepts checkpoints of the stock torch optimizers, which may lack ``initial_lr`` (ref:974-986)."""
@@ -459,6 +594,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         """Inverse of :meth:`get_fp32_model_state_dict`: narrows into the parameters and recomputes their ECC
         (ref:1086-1147)."""
         module = cast(nn.Module, model.module if hasattr(model, "module") else model)
+        self._plan_epoch += 1  # error_bits tensors are replaced below
         for name, param in module.named_parameters():
             if name not in fp32_state_dict:
                 continue

@@ -3,12 +3,11 @@
 from __future__ import annotations
 
 from collections.abc import Iterable
-from typing import Literal, Optional
+from typing import Any, Literal, Optional
 
 import torch
 
-from .base import FlashOptimizer, LaunchKey
-from .launcher import StepTensors
+from .base import FlashOptimizer
 from .state import QuantizedTensorSpec
 
 
@@ -53,18 +52,16 @@ class FlashLion(FlashOptimizer):
     def _quantized_state_spec(self) -> dict[str, QuantizedTensorSpec]:
         return {"exp_avg": QuantizedTensorSpec(signed=True)}
 
-    def _plan_step(self, param, grad, errors, param_state, hparams) -> Optional[tuple[LaunchKey, StepTensors]]:
+    def _kernel_kind(self, hparams: dict[str, Any]) -> str:
+        return "momentum"
+
+    def _moment_names(self, kind: str) -> tuple[Optional[str], Optional[str]]:
+        return "exp_avg", None
+
+    def _kernel_scalars(self, hparams: dict[str, Any], step: Optional[int]) -> dict[str, Any]:
         lr = hparams["lr"]
         weight_decay = hparams["weight_decay"]  # ref:1290-1294
         weight_decay *= (lr / hparams["initial_lr"]) if self._decouple_lr else lr
-        if errors is not None and errors.dtype not in (torch.int8, torch.int16):
-            raise ValueError("Errors needs to be int8 or int16")
-        mom = param_state["exp_avg"]
-        beta1, beta2 = hparams["betas"][0], hparams["betas"][1]
         # the kernel's momentum decay is beta2, its update interpolation beta1 (ref:1313-1317)
-        scalars = (
-            ("lr", lr), ("mom_coef", beta2), ("update_coef", beta1), ("weight_decay", weight_decay),
-            ("decoupled", False), ("nesterov", False), ("do_lion", True),
-        )
-        return (LaunchKey("momentum", param.dtype, 0 if errors is None else errors.element_size(), mom.is_quantized(), scalars),
-                StepTensors(param=param, grad=grad, ecc=errors, mom=mom.kernel_tensor, mom_scales=mom.kernel_scales_or_self))
+        return dict(lr=lr, mom_coef=hparams["betas"][1], update_coef=hparams["betas"][0], weight_decay=weight_decay,
+                    decoupled=False, nesterov=False, do_lion=True)

@@ -3,12 +3,11 @@
 from __future__ import annotations
 
 from collections.abc import Iterable
-from typing import Literal, Optional
+from typing import Any, Literal, Optional
 
 import torch
 
-from .base import FlashOptimizer, LaunchKey
-from .launcher import StepTensors
+from .base import FlashOptimizer
 from .state import QuantizedTensorSpec
 
 
@@ -59,26 +58,23 @@ class FlashSGD(FlashOptimizer):
             return {"momentum_buffer": QuantizedTensorSpec(signed=True)}
         return {}
 
-    def _plan_step(self, param, grad, errors, param_state, hparams) -> Optional[tuple[LaunchKey, StepTensors]]:
+    def _kernel_kind(self, hparams: dict[str, Any]) -> str:
+        # without momentum no buffer exists: the momentum-free kernel steps the weights directly (the reference
+        # handles this case in eager ops, ref:1447-1465)
+        return "plain" if hparams["momentum"] == 0.0 else "momentum"
+
+    def _moment_names(self, kind: str) -> tuple[Optional[str], Optional[str]]:
+        return ("momentum_buffer" if kind == "momentum" else None), None
+
+    def _kernel_scalars(self, hparams: dict[str, Any], step: Optional[int]) -> dict[str, Any]:
         lr = hparams["lr"]
-        momentum = hparams["momentum"]
         weight_decay = hparams["weight_decay"]
         if self._decoupled:  # ref:1438-1442
             weight_decay *= (lr / hparams["initial_lr"]) if self._decouple_lr else lr
-        ecc_bytes = 0 if errors is None else errors.element_size()
-        if momentum == 0.0:
-            # no buffer exists: the momentum-free kernel (the reference handles this case in eager ops, ref:1447-1465)
-            scalars = (("lr", lr), ("weight_decay", weight_decay), ("decoupled", self._decoupled))
-            return (LaunchKey("plain", param.dtype, ecc_bytes, False, scalars),
-                    StepTensors(param=param, grad=grad, ecc=errors, mom=None, mom_scales=None))
-        buf = param_state["momentum_buffer"]
-        scalars = (
-            ("lr", lr), ("mom_coef", momentum), ("update_coef", 1.0 - hparams["dampening"]),
-            ("weight_decay", weight_decay), ("decoupled", self._decoupled), ("nesterov", self._nesterov),
-            ("do_lion", False),
-        )
-        return (LaunchKey("momentum", param.dtype, ecc_bytes, buf.is_quantized(), scalars),
-                StepTensors(param=param, grad=grad, ecc=errors, mom=buf.kernel_tensor, mom_scales=buf.kernel_scales_or_self))
+        if hparams["momentum"] == 0.0:
+            return dict(lr=lr, weight_decay=weight_decay, decoupled=self._decoupled)
+        return dict(lr=lr, mom_coef=hparams["momentum"], update_coef=1.0 - hparams["dampening"],
+                    weight_decay=weight_decay, decoupled=self._decoupled, nesterov=self._nesterov, do_lion=False)
 
 
 class FlashSGDW(FlashSGD):

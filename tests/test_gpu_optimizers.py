@@ -652,3 +652,46 @@ def test_ecc_invariants_over_every_binade():
             for e in exps:
                 for inv, c in zip(names, counts(sign, e, dtype)):
                     assert c <= budget.get((name, inv), 0), (name, sign, e, inv, c)
+
+
+# ------------------------------------------------------------------------------- cached step() plans
+
+
+def test_cached_step_plan_follows_moving_missing_and_freed_gradients():
+    """step() caches a group's launch tables after the first call.  The cache must notice gradients that were
+    re-allocated at other addresses, fall back when a gradient is missing, never keep a freed gradient alive, and
+    stay bit-identical to per-tensor stepping throughout."""
+    import gc
+    import weakref
+
+    fo = _fo()
+    shapes = [5000, 33, 4096, 70001]
+    pa, pb = _make_params(shapes, torch.bfloat16, 21), _make_params(shapes, torch.bfloat16, 21)
+    oa, ob = fo.FlashAdamW(pa, lr=1e-3), fo.FlashAdamW(pb, lr=1e-3)
+    hold = []
+    for it in range(6):
+        _set_grads(pa, 100 + it)
+        _set_grads(pb, 100 + it)
+        if it == 2:                       # keep the old gradients alive so the new ones land elsewhere
+            hold = [p.grad for p in pa]
+            _set_grads(pa, 100 + it)
+            assert any(p.grad.data_ptr() != h.data_ptr() for p, h in zip(pa, hold))
+        if it == 4:                       # one parameter without a gradient this step
+            pa[1].grad = None
+            pb[1].grad = None
+        if it == 3:
+            oa.param_groups[0]["lr"] = ob.param_groups[0]["lr"] = 5e-4   # scheduler-style change
+        oa.step()
+        for p in pb:
+            ob.step_param(p)
+    for a, b in zip(pa, pb):
+        assert torch.equal(a, b)
+        sa, sb = _state_tensors(oa, a), _state_tensors(ob, b)
+        for k in sa:
+            assert parity.bits_equal(sa[k], sb[k]), k
+    assert oa.state[pa[0]]["step"].item() == 6 and oa.state[pa[1]]["step"].item() == 5
+    ref = weakref.ref(pa[0].grad)
+    oa.zero_grad(set_to_none=True)
+    del hold
+    gc.collect()
+    assert ref() is None, "the optimizer's cached plan kept a gradient alive"
