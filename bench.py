@@ -18,6 +18,8 @@ Workloads (``--workload``):
   llama8b-fp32-release
                   fp32 parameters, quantised moments, one launch per tensor in reverse order as under gradient
                   release; ends with a compressed state_dict save -> load round trip checked bit for bit.
+  copy            4 GiB device copy with the library's copy kernel: calibrates the rocprof byte counters and shows
+                  the attainable read+write rate (``value`` is meaningless here, read ``roofline``).
 
 Reported: ``value`` = parameters updated per second; ``roofline`` = algorithmic HBM bytes of one step divided
 by the average duration of a step measured with events on the launch stream, against the 8 TB/s peak;
@@ -145,6 +147,16 @@ def build_workload(name: str, device):
                          "per tensor in reverse order as under gradient release",
                     launch="one single-tensor launch per tensor (291 per step)", optimizer="FlashAdamW", mwb=None,
                     checkpoint_roundtrip=True)
+    if name == "copy":
+        from flashoptim_amd.kernels import copy_bytes
+
+        n = 1 << 32
+        src = torch.empty(n, dtype=torch.uint8, device=device).random_(0, 255)
+        dst = torch.empty_like(src)
+        holder = torch.nn.Parameter(src.view(torch.float32)[:0])  # no parameters: this workload only moves bytes
+        return dict(params=[holder], opt=None, step=lambda: copy_bytes(dst, src), bpp=0.0, copy_bytes=2 * n,
+                    desc="device copy of 4 GiB with the library's copy kernel (counter calibration, attainable rate)",
+                    launch="one copy launch per step", optimizer=None, mwb=None)
     raise SystemExit(f"unknown workload {name!r}")
 
 
@@ -239,7 +251,7 @@ def main() -> None:
     device_ms = sorted(a.elapsed_time(b) for a, b in events)
     avg_device_ms = sum(device_ms) / len(device_ms)
 
-    step_bytes = total * work["bpp"]
+    step_bytes = work.get("copy_bytes", total * work["bpp"])
     achieved = step_bytes / (avg_device_ms * 1e-3) / 1e9
     out = {
         "metric": "params updated/sec + achieved HBM GB/s (% peak), FlashAdamW step on 8B params",
