@@ -13,6 +13,8 @@ Workloads (``--workload``):
                   headline metric is quoted on.
   llama8b-mwb32   same shapes, master_weight_bits=32 (int16 correction term).
   flat-2p30       one flat bf16 tensor of 2^30 elements, FlashAdamW, master_weight_bits=24.
+  llama8b-lion / llama8b-sgdw
+                  the same parameter list under FlashLion / FlashSGDW (one quantised moment), master_weight_bits=24.
   ragged-lion / ragged-sgdw
                   4096 bf16 tensors with log-uniform lengths in [1, 2^24] (~1e9 parameters), FlashLion / FlashSGDW.
   llama8b-fp32-release
@@ -107,6 +109,18 @@ def build_workload(name: str, device):
         return dict(params=params, opt=opt, step=opt.step, bpp=bytes_per_param(2, 1 if mwb == 24 else 2, 2),
                     desc=f"Llama-3-8B-shaped parameter list, bf16, FlashAdamW, master_weight_bits={mwb}",
                     launch="one multi-tensor launch per step", optimizer="FlashAdamW", mwb=mwb)
+    if name in ("llama8b-lion", "llama8b-sgdw"):
+        shapes = llama3_8b_shapes()
+        g = torch.Generator().manual_seed(2)
+        scales = (10.0 ** (torch.rand(len(shapes), generator=g) * 2 - 1)).tolist()
+        params = make_params(shapes, torch.bfloat16, device, scales)
+        if name == "llama8b-lion":
+            opt = fo.FlashLion(params, lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1, master_weight_bits=24)
+        else:
+            opt = fo.FlashSGDW(params, momentum=0.9, lr=1e-2, weight_decay=1e-4, master_weight_bits=24)
+        return dict(params=params, opt=opt, step=opt.step, bpp=bytes_per_param(2, 1, 1),
+                    desc=f"Llama-3-8B-shaped parameter list, bf16, {type(opt).__name__}, master_weight_bits=24",
+                    launch="one multi-tensor launch per step", optimizer=type(opt).__name__, mwb=24)
     if name == "flat-2p30":
         params = make_params([("flat", (1 << 30,))], torch.bfloat16, device)
         opt = fo.FlashAdamW(params, master_weight_bits=24, **hp)

@@ -19,53 +19,67 @@ struct AdamHyper {
     float den_scale, den_bias;
 };
 
-template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool FAST>
-__device__ __forceinline__ void adam_lane(const TensorPtrs& t, int64_t first, const AdamHyper& h, const float* lut_lane) {
+// What a lane holds between issuing its loads and consuming them.
+template <int DT, int ECCB, bool QUANT> struct AdamRaw {
+    static constexpr int EPL = DTypeInfo<DT>::epl;
+    Pack<DTypeInfo<DT>::bytes, EPL> p, g;
+    Pack<ECCB, EPL> e;
+    Pack<QUANT ? 1 : DTypeInfo<DT>::bytes, EPL> m, v;
+    uint16_t sm, sv;
+};
+
+template <int DT, int ECCB, bool QUANT, int FAST>
+__device__ __forceinline__ void adam_load(const TensorPtrs& t, int64_t first, AdamRaw<DT, ECCB, QUANT>& r) {
     constexpr int EPL = DTypeInfo<DT>::epl;
     constexpr int PB = DTypeInfo<DT>::bytes;
     constexpr int SB = QUANT ? 1 : PB;  // state bytes per element
     const int64_t n = t.n;
-
-    Pack<PB, EPL> praw, graw;
-    Pack<ECCB, EPL> eraw;
-    Pack<SB, EPL> mraw, vraw;
-    load_lane<PB, EPL, FAST>(graw, t.grad, first, n);
-    load_lane<PB, EPL, FAST>(praw, t.param, first, n);
-    load_lane<ECCB, EPL, FAST>(eraw, t.ecc, first, n);
-    load_lane<SB, EPL, FAST>(mraw, t.mom, first, n);
-    load_lane<SB, EPL, FAST>(vraw, t.var, first, n);
-    const bool live_group = FAST || first < n;  // the lane owns at least one real element
-    const int64_t group = first >> 5;
-    float sm = 1.0f, sv = 1.0f;  // masked scales read 1.0 (ref:2318-2323)
+    load_lane<PB, EPL, FAST>(r.g, t.grad, first, n);
+    load_lane<PB, EPL, FAST>(r.p, t.param, first, n);
+    load_lane<ECCB, EPL, FAST>(r.e, t.ecc, first, n);
+    load_lane<SB, EPL, FAST>(r.m, t.mom, first, n);
+    load_lane<SB, EPL, FAST>(r.v, t.var, first, n);
+    r.sm = r.sv = 0x3c00;  // masked scales read 1.0 (ref:2318-2323)
     if constexpr (QUANT) {
-        if (live_group) {
-            sm = f16_bits_to_f32(t.mom_scales[group]);
-            sv = f16_bits_to_f32(t.var_scales[group]);
+        if (FAST == kVector || first < n) {
+            r.sm = t.mom_scales[first >> 5];
+            r.sv = t.var_scales[first >> 5];
         }
     }
+}
+
+template <int DT, int ECCB, bool QUANT, bool DECOUPLED, int FAST>
+__device__ __forceinline__ void adam_finish(const TensorPtrs& t, int64_t first, AdamRaw<DT, ECCB, QUANT>& raw,
+                                            const AdamHyper& h, const float* lut_lane) {
+    constexpr int EPL = DTypeInfo<DT>::epl;
+    constexpr int PB = DTypeInfo<DT>::bytes;
+    constexpr int SB = QUANT ? 1 : PB;
+    const int64_t n = t.n;
+    const bool live_group = FAST == kVector || first < n;  // the lane owns at least one real element
+    const int64_t group = first >> 5;
     // the EMA decay is folded into the group scale: one multiply per lane instead of one per element
-    const float sm_b1 = sm * h.b1;
-    const float sv_b2 = sv * h.sqrt_b2_over_255;
+    const float sm_b1 = f16_bits_to_f32(raw.sm) * h.b1;
+    const float sv_b2 = f16_bits_to_f32(raw.sv) * h.sqrt_b2_over_255;
 
     float p[EPL], m[EPL], r[EPL], v[EPL];
-    read_master<DT, ECCB, EPL>(p, praw, eraw);
+    read_master<DT, ECCB, EPL>(p, raw.p, raw.e);
 
     float am = 0.0f, vm = 0.0f;
 #pragma unroll
     for (int k = 0; k < EPL; ++k) {
-        float g = widen<DT, EPL>(graw, k);
+        float g = widen<DT, EPL>(raw.g, k);
         if constexpr (!DECOUPLED) g = g + p[k] * h.wd;                              // ref:2310-2311
         float mn, vn;
         if constexpr (QUANT) {
             // m = dequant(m) * b1 + g * (1 - b1)   (ref:2332-2343, 2357)
-            mn = fmaf(StepLut::lookup(lut_lane, byte_of<EPL>(mraw, k)), sm_b1, g * h.one_m_b1);
+            mn = fmaf(StepLut::lookup(lut_lane, byte_of<EPL>(raw.m, k)), sm_b1, g * h.one_m_b1);
             // v = dequant(v) * b2 + g^2 * (1 - b2), dequant(v) = (code/255 * scale)^2   (ref:2333-2348, 2360)
-            const float s = (float)byte_of<EPL>(vraw, k) * sv_b2;
+            const float s = (float)byte_of<EPL>(raw.v, k) * sv_b2;
             vn = fmaf(s, s, (g * g) * h.one_m_b2);
         } else {
             // unquantised states: operation by operation as written in the reference, no contraction
-            mn = widen<DT, EPL>(mraw, k) * h.b1 + g * h.one_m_b1;                   // ref:2351-2357
-            vn = widen<DT, EPL>(vraw, k) * h.b2 + (g * g) * h.one_m_b2;             // ref:2360
+            mn = widen<DT, EPL>(raw.m, k) * h.b1 + g * h.one_m_b1;                   // ref:2351-2357
+            vn = widen<DT, EPL>(raw.v, k) * h.b2 + (g * g) * h.one_m_b2;             // ref:2360
         }
         float pk = p[k];
         if constexpr (DECOUPLED) pk = pk * h.one_m_wd;                              // ref:2363-2364
@@ -74,13 +88,16 @@ __device__ __forceinline__ void adam_lane(const TensorPtrs& t, int64_t first, co
         const float den = fmaf(rk, h.den_scale, h.den_bias);
         pk = fmaf(-mn, __builtin_amdgcn_rcpf(den), pk);
         p[k] = pk; m[k] = mn; r[k] = rk; v[k] = vn;
-        am = fmaxf(am, fabsf(mn));
-        vm = fmaxf(vm, vn);
+    }
+#pragma unroll
+    for (int k = 0; k < EPL; k += 2) {  // pairs, so that each step is one three-operand max
+        am = fmaxf(fmaxf(am, fabsf(m[k])), fabsf(m[k + 1]));
+        vm = fmaxf(fmaxf(vm, v[k]), v[k + 1]);
     }
 
     Pack<ECCB, EPL> eout;
-    write_master<DT, ECCB, EPL>(p, praw, eout);
-    store_lane<PB, EPL, FAST>(praw, t.param, first, n);
+    write_master<DT, ECCB, EPL>(p, raw.p, eout);
+    store_lane<PB, EPL, FAST>(raw.p, t.param, first, n);
     store_lane<ECCB, EPL, FAST>(eout, t.ecc, first, n);
 
     if constexpr (QUANT) {
@@ -88,29 +105,36 @@ __device__ __forceinline__ void adam_lane(const TensorPtrs& t, int64_t first, co
         // root of max(v)
         am = fmaxf(group_max<EPL>(am), 1e-12f);
         const float av = fmaxf(sqrt_rn(group_max<EPL>(vm)), 1e-12f);
-        quantize_mom<EPL>(m, am, mraw);
-        quantize_var<EPL>(r, av, vraw);
-        store_lane<1, EPL, FAST>(mraw, t.mom, first, n);
-        store_lane<1, EPL, FAST>(vraw, t.var, first, n);
+        quantize_mom<EPL>(m, am, raw.m);
+        quantize_var<EPL>(r, av, raw.v);
+        store_lane<1, EPL, FAST>(raw.m, t.mom, first, n);
+        store_lane<1, EPL, FAST>(raw.v, t.var, first, n);
         if (live_group && (threadIdx.x & (32 / EPL - 1)) == 0) {                    // ref:2424-2434
             t.mom_scales[group] = f32_to_f16_bits(am);
             t.var_scales[group] = f32_to_f16_bits(av);
         }
     } else {
-        narrow_all<DT, EPL>(m, mraw);                                               // ref:2435-2438
-        narrow_all<DT, EPL>(v, vraw);
-        store_lane<SB, EPL, FAST>(mraw, t.mom, first, n);
-        store_lane<SB, EPL, FAST>(vraw, t.var, first, n);
+        narrow_all<DT, EPL>(m, raw.m);                                              // ref:2435-2438
+        narrow_all<DT, EPL>(v, raw.v);
+        store_lane<SB, EPL, FAST>(raw.m, t.mom, first, n);
+        store_lane<SB, EPL, FAST>(raw.v, t.var, first, n);
     }
 }
 
 template <int DT, int ECCB, bool QUANT, bool DECOUPLED> struct AdamOp {
     using Hyper = AdamHyper;
     static constexpr bool kNeedsLut = QUANT;
+    // measured optima on MI355X for the 8B-parameter step (2-byte parameters: 3.6-4.5 KiB of loads per wavefront;
+    // fp32 parameters: 2.5 KiB)
+    static constexpr int kResidentWorkgroups = DT == DT_F32 ? 16 : 14;
     static constexpr int kEpl = DTypeInfo<DT>::epl;
-    template <bool FAST>
-    __device__ __forceinline__ static void lane(const TensorPtrs& t, int64_t first, const Hyper& h, const float* lut) {
-        adam_lane<DT, ECCB, QUANT, DECOUPLED, FAST>(t, first, h, lut);
+    using Raw = AdamRaw<DT, ECCB, QUANT>;
+    template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, int64_t first, Raw& r) {
+        adam_load<DT, ECCB, QUANT, FAST>(t, first, r);
+    }
+    template <int FAST>
+    __device__ __forceinline__ static void finish(const TensorPtrs& t, int64_t first, Raw& r, const Hyper& h, const float* lut) {
+        adam_finish<DT, ECCB, QUANT, DECOUPLED, FAST>(t, first, r, h, lut);
     }
 };
 

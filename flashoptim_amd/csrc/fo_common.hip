@@ -47,8 +47,12 @@ static int env_int(const char* name, int fallback) {
     return (v >= 1 && v <= 1024) ? v : fallback;
 }
 
-int tiles_per_block() {
-    static const int value = env_int("FO_TILES_PER_BLOCK", 1);
+int step_lds_pad_bytes() {
+    static const int value = [] {
+        const char* e = getenv("FO_STEP_LDS_PAD");
+        const int v = e ? atoi(e) : -1;
+        return (v >= 0 && v <= 64 * 1024) ? v : -1;
+    }();
     return value;
 }
 

@@ -16,6 +16,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "../../include/flashoptim_hip.h"
+
 namespace fo {
 
 typedef uint32_t u32;
@@ -26,7 +28,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kGroup = 32;             // ref:1549, 2219: quantisation group
-constexpr int kTileElems = 4096;       // unit of the multi-tensor chunk table (FO_TILE_ELEMS)
+constexpr int kTileElems = FO_TILE_ELEMS;  // unit of scheduling and of the multi-tensor chunk table (4096)
 constexpr float kMagic = 12582912.0f;  // 1.5 * 2^23: x + kMagic leaves rne(x) in the low mantissa bits
 
 enum { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2 };
@@ -118,16 +120,35 @@ __device__ __forceinline__ void store_guarded(const Pack<EB, EPL>& d, void* base
         }
     }
 }
-template <int EB, int EPL, bool FAST>
+// How a lane reaches its EPL elements of a stream:
+//   kVector   one vector access, no checks (the whole span is in range and every stream is 16-byte aligned);
+//   kLane     aligned streams, span cut by the end of the tensor: lanes that are entirely in range still use the
+//             vector access, only the lane that straddles the end goes element by element;
+//   kGuarded  element by element (unaligned views).
+enum { kGuarded = 0, kVector = 1, kLane = 2 };
+
+template <int EB, int EPL, int MODE>
 __device__ __forceinline__ void load_lane(Pack<EB, EPL>& d, const void* base, int64_t first, int64_t n) {
     if constexpr (EB > 0) {
-        if constexpr (FAST) load_vec<EB, EPL>(d, base, first); else load_guarded<EB, EPL>(d, base, first, n);
+        if constexpr (MODE == kVector) {
+            load_vec<EB, EPL>(d, base, first);
+        } else if constexpr (MODE == kLane) {
+            if (first + EPL <= n) load_vec<EB, EPL>(d, base, first); else load_guarded<EB, EPL>(d, base, first, n);
+        } else {
+            load_guarded<EB, EPL>(d, base, first, n);
+        }
     }
 }
-template <int EB, int EPL, bool FAST>
+template <int EB, int EPL, int MODE>
 __device__ __forceinline__ void store_lane(const Pack<EB, EPL>& d, void* base, int64_t first, int64_t n) {
     if constexpr (EB > 0) {
-        if constexpr (FAST) store_vec<EB, EPL>(d, base, first); else store_guarded<EB, EPL>(d, base, first, n);
+        if constexpr (MODE == kVector) {
+            store_vec<EB, EPL>(d, base, first);
+        } else if constexpr (MODE == kLane) {
+            if (first + EPL <= n) store_vec<EB, EPL>(d, base, first); else store_guarded<EB, EPL>(d, base, first, n);
+        } else {
+            store_guarded<EB, EPL>(d, base, first, n);
+        }
     }
 }
 
@@ -204,16 +225,26 @@ template <int DT, int ECCB> __device__ __forceinline__ float ecc_join(float wide
 //   is exact; the only tie that can occur is +-63.5, where half-even and half-away agree.  One fma against
 //   1.5 * 2^23 then leaves the rounded integer in the low mantissa bits.
 //   CLAMP = false is for callers whose narrow value IS the round-to-nearest of p (|en| <= 1 by construction).
+//   For them the bf16/int8 case folds the scaling into the fma: with eb the biased exponent field of the narrow
+//   value (1..254), en * 127 = err * 127 * 2^(135 - eb).  That factor can exceed the fp32 range, so both fma
+//   operands carry an extra 2^-13: S = 127 * 2^(122 - eb) is a normal number for every eb (bit pattern
+//   0x7ffe0000 - (eb << 23)) and 1.5 * 2^10 + en * 127 * 2^-13 has the same mantissa bits as
+//   1.5 * 2^23 + en * 127, rounded at the same place.
 template <int DT, int ECCB, bool CLAMP> __device__ __forceinline__ u32 ecc_split_bits(float p, float widened) {
     const float err = p - widened;
-    const int nls = (DTypeInfo<DT>::mant + 1 + 127) - (int)(pow2_of_exponent_bits<DT>(widened) >> 23);
-    float en = __builtin_amdgcn_ldexpf(err, nls);
-    if constexpr (CLAMP) en = __builtin_amdgcn_fmed3f(en, -1.0f, 1.0f);
-    if constexpr (DT == DT_BF16 && ECCB == 1) {
-        return as_u32(fmaf(en, EccInfo<ECCB>::max_val, kMagic));
+    if constexpr (DT == DT_BF16 && ECCB == 1 && !CLAMP) {
+        const float s = as_f32(0x7ffe0000u - pow2_of_exponent_bits<DT>(widened));
+        return as_u32(fmaf(err, s, 1536.0f));
     } else {
-        const float sc = en * EccInfo<ECCB>::max_val;
-        return (u32)(int)(sc + __builtin_copysignf(0.5f, sc));
+        const int nls = (DTypeInfo<DT>::mant + 1 + 127) - (int)(pow2_of_exponent_bits<DT>(widened) >> 23);
+        float en = __builtin_amdgcn_ldexpf(err, nls);
+        if constexpr (CLAMP) en = __builtin_amdgcn_fmed3f(en, -1.0f, 1.0f);
+        if constexpr (DT == DT_BF16 && ECCB == 1) {
+            return as_u32(fmaf(en, EccInfo<ECCB>::max_val, kMagic));
+        } else {
+            const float sc = en * EccInfo<ECCB>::max_val;
+            return (u32)(int)(sc + __builtin_copysignf(0.5f, sc));
+        }
     }
 }
 
@@ -268,16 +299,29 @@ struct SoftsignTable {
 __device__ const SoftsignTable kSoftsignTable = SoftsignTable();
 
 // The table lives in LDS during a kernel.  REPL copies per entry; a lane uses copy (lane % REPL).
-// REPL = 32 gives every lane its own bank (entry b, lane l at [b*32 + (l & 31)]): no bank conflicts.
-template <int REPL> struct Lut {
+// REPL = 32 would give every lane its own bank; REPL = 1 (1 KiB) costs a few conflicted reads but fills with
+// one store per thread, which matters because every short-lived workgroup fills its own copy.
+// Filling is split so that the global read of the table is in flight together with the workgroup's streaming
+// loads: fetch() first, commit() (LDS stores + barrier) just before the first lookup.  T = workgroup size.
+template <int REPL, int T> struct Lut {
     static constexpr int kFloats = 256 * REPL;
-    __device__ __forceinline__ static void build(float* lut) {
-        for (int b = threadIdx.x; b < 256; b += blockDim.x) {
-            const float v = kSoftsignTable.v[b];
+    static constexpr int kPerThread = T >= 256 ? 1 : 256 / T;  // table entries a thread copies
+    struct Frag { float v[kPerThread]; };
+    __device__ __forceinline__ static Frag fetch() {
+        Frag f;
+        const float* src = kSoftsignTable.v + (threadIdx.x & (256 / kPerThread - 1)) * kPerThread;
 #pragma unroll
-            for (int i = 0; i < REPL; ++i) lut[b * REPL + i] = v;
+        for (int j = 0; j < kPerThread; ++j) f.v[j] = src[j];
+        return f;
+    }
+    __device__ __forceinline__ static void commit(float* lut, const Frag& f) {
+        if (T <= 256 || threadIdx.x < 256) {
+#pragma unroll
+            for (int j = 0; j < kPerThread; ++j)
+#pragma unroll
+                for (int i = 0; i < REPL; ++i) lut[(threadIdx.x * kPerThread + j) * REPL + i] = f.v[j];
         }
-        __syncthreads();
+        __syncthreads();  // a single-wavefront workgroup needs no hardware barrier; the compiler drops it
     }
     __device__ __forceinline__ static const float* lane_base(const float* lut) { return lut + (threadIdx.x & (REPL - 1)); }
     __device__ __forceinline__ static float lookup(const float* lane_lut, u32 byte) { return lane_lut[byte * REPL]; }

@@ -15,10 +15,9 @@ int check_hip(hipError_t e, const char* what);
 int compute_units();
 const char* last_error();
 
-// Tiles (4096 elements each) a block of the single-tensor kernels walks before it retires.  Small enough that
-// the launch is one pass of many short-lived blocks, large enough to amortise the per-block table set-up.
-// FO_TILES_PER_BLOCK in the environment overrides it (read once; for tuning).
-int tiles_per_block();
+// Override, from FO_STEP_LDS_PAD in the environment, of the unused dynamic LDS that every step-kernel workgroup
+// requests to bound the workgroups resident on a compute unit; -1 when unset (read once; for tuning).
+int step_lds_pad_bytes();
 
 // Tiles per work item of the multi-tensor chunk table when the caller passes tiles_per_chunk <= 0.
 // FO_TILES_PER_CHUNK in the environment overrides it (read once; for tuning).

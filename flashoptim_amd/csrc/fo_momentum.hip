@@ -15,34 +15,49 @@ struct MomentumHyper {
     int apply_decay;  // momentum-free branch only: the reference skips both decays when weight_decay == 0
 };
 
-template <int DT, int ECCB, bool QUANT, int KIND, bool FAST>
-__device__ __forceinline__ void momentum_lane(const TensorPtrs& t, int64_t first, const MomentumHyper& h, const float* lut_lane) {
+template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumRaw {
+    static constexpr int EPL = DTypeInfo<DT>::epl;
+    static constexpr int SB = (KIND == KIND_PLAIN) ? 0 : (QUANT ? 1 : DTypeInfo<DT>::bytes);
+    Pack<DTypeInfo<DT>::bytes, EPL> p, g;
+    Pack<ECCB, EPL> e;
+    Pack<SB, EPL> m;
+    uint16_t sm;
+};
+
+template <int DT, int ECCB, bool QUANT, int KIND, int FAST>
+__device__ __forceinline__ void momentum_load(const TensorPtrs& t, int64_t first, MomentumRaw<DT, ECCB, QUANT, KIND>& r) {
     constexpr int EPL = DTypeInfo<DT>::epl;
     constexpr int PB = DTypeInfo<DT>::bytes;
-    constexpr int SB = (KIND == KIND_PLAIN) ? 0 : (QUANT ? 1 : PB);
+    constexpr int SB = MomentumRaw<DT, ECCB, QUANT, KIND>::SB;
     const int64_t n = t.n;
-
-    Pack<PB, EPL> praw, graw;
-    Pack<ECCB, EPL> eraw;
-    Pack<SB, EPL> mraw;
-    load_lane<PB, EPL, FAST>(graw, t.grad, first, n);
-    load_lane<PB, EPL, FAST>(praw, t.param, first, n);
-    load_lane<ECCB, EPL, FAST>(eraw, t.ecc, first, n);
-    load_lane<SB, EPL, FAST>(mraw, t.mom, first, n);
-    const bool live_group = FAST || first < n;
-    const int64_t group = first >> 5;
-    float sm = 1.0f;
+    load_lane<PB, EPL, FAST>(r.g, t.grad, first, n);
+    load_lane<PB, EPL, FAST>(r.p, t.param, first, n);
+    load_lane<ECCB, EPL, FAST>(r.e, t.ecc, first, n);
+    load_lane<SB, EPL, FAST>(r.m, t.mom, first, n);
+    r.sm = 0x3c00;  // 1.0
     if constexpr (QUANT && KIND != KIND_PLAIN) {
-        if (live_group) sm = f16_bits_to_f32(t.mom_scales[group]);                  // ref:1645-1646
+        if (FAST == kVector || first < n) r.sm = t.mom_scales[first >> 5];                     // ref:1645-1646
     }
+}
+
+template <int DT, int ECCB, bool QUANT, int KIND, int FAST>
+__device__ __forceinline__ void momentum_finish(const TensorPtrs& t, int64_t first, MomentumRaw<DT, ECCB, QUANT, KIND>& raw,
+                                                const MomentumHyper& h, const float* lut_lane) {
+    constexpr int EPL = DTypeInfo<DT>::epl;
+    constexpr int PB = DTypeInfo<DT>::bytes;
+    constexpr int SB = MomentumRaw<DT, ECCB, QUANT, KIND>::SB;
+    const int64_t n = t.n;
+    const bool live_group = FAST == kVector || first < n;
+    const int64_t group = first >> 5;
+    const float sm = f16_bits_to_f32(raw.sm);
 
     float p[EPL], m[EPL];
-    read_master<DT, ECCB, EPL>(p, praw, eraw);
+    read_master<DT, ECCB, EPL>(p, raw.p, raw.e);
 
     float am = 0.0f;
 #pragma unroll
     for (int k = 0; k < EPL; ++k) {
-        float g = widen<DT, EPL>(graw, k);
+        float g = widen<DT, EPL>(raw.g, k);
         float pk = p[k];
         if constexpr (KIND == KIND_PLAIN) {
             if (h.apply_decay && !h.decoupled) g = g + pk * h.wd;                   // ref:1452-1453
@@ -51,8 +66,8 @@ __device__ __forceinline__ void momentum_lane(const TensorPtrs& t, int64_t first
         } else {
             if (KIND == KIND_SGD && !h.decoupled) g = g + pk * h.wd;                // ref:1639-1640
             float mo;
-            if constexpr (QUANT) mo = StepLut::lookup(lut_lane, byte_of<EPL>(mraw, k)) * sm;   // ref:1648-1657
-            else mo = widen<DT, EPL>(mraw, k);                                      // ref:1660-1661
+            if constexpr (QUANT) mo = StepLut::lookup(lut_lane, byte_of<EPL>(raw.m, k)) * sm;   // ref:1648-1657
+            else mo = widen<DT, EPL>(raw.m, k);                                     // ref:1660-1661
             float mn;
             if constexpr (KIND == KIND_LION) {
                 const float u = (mo * h.update_coef) + (g * h.one_m_update_coef);        // ref:1667
@@ -67,25 +82,29 @@ __device__ __forceinline__ void momentum_lane(const TensorPtrs& t, int64_t first
                 else pk = pk - mn * h.lr;                                                // ref:1682-1683
             }
             m[k] = mn;
-            am = fmaxf(am, fabsf(mn));
         }
         p[k] = pk;
     }
 
+    if constexpr (KIND != KIND_PLAIN) {
+#pragma unroll
+        for (int k = 0; k < EPL; k += 2) am = fmaxf(fmaxf(am, fabsf(m[k])), fabsf(m[k + 1]));
+    }
+
     Pack<ECCB, EPL> eout;
-    write_master<DT, ECCB, EPL>(p, praw, eout);                                     // ref:1684-1694
-    store_lane<PB, EPL, FAST>(praw, t.param, first, n);
+    write_master<DT, ECCB, EPL>(p, raw.p, eout);                                    // ref:1684-1694
+    store_lane<PB, EPL, FAST>(raw.p, t.param, first, n);
     store_lane<ECCB, EPL, FAST>(eout, t.ecc, first, n);
 
     if constexpr (KIND != KIND_PLAIN) {
         if constexpr (QUANT) {
             am = fmaxf(group_max<EPL>(am), 1e-12f);                                 // ref:1702-1703
-            quantize_mom<EPL>(m, am, mraw);
-            store_lane<1, EPL, FAST>(mraw, t.mom, first, n);
+            quantize_mom<EPL>(m, am, raw.m);
+            store_lane<1, EPL, FAST>(raw.m, t.mom, first, n);
             if (live_group && (threadIdx.x & (32 / EPL - 1)) == 0) t.mom_scales[group] = f32_to_f16_bits(am);  // ref:1713-1716
         } else {
-            narrow_all<DT, EPL>(m, mraw);                                           // ref:1717-1719
-            store_lane<SB, EPL, FAST>(mraw, t.mom, first, n);
+            narrow_all<DT, EPL>(m, raw.m);                                          // ref:1717-1719
+            store_lane<SB, EPL, FAST>(raw.m, t.mom, first, n);
         }
     }
 }
@@ -93,10 +112,15 @@ __device__ __forceinline__ void momentum_lane(const TensorPtrs& t, int64_t first
 template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumOp {
     using Hyper = MomentumHyper;
     static constexpr bool kNeedsLut = QUANT && KIND != KIND_PLAIN;
+    static constexpr int kResidentWorkgroups = 20;  // measured optimum on MI355X (3 KiB of loads per wavefront)
     static constexpr int kEpl = DTypeInfo<DT>::epl;
-    template <bool FAST>
-    __device__ __forceinline__ static void lane(const TensorPtrs& t, int64_t first, const Hyper& h, const float* lut) {
-        momentum_lane<DT, ECCB, QUANT, KIND, FAST>(t, first, h, lut);
+    using Raw = MomentumRaw<DT, ECCB, QUANT, KIND>;
+    template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, int64_t first, Raw& r) {
+        momentum_load<DT, ECCB, QUANT, KIND, FAST>(t, first, r);
+    }
+    template <int FAST>
+    __device__ __forceinline__ static void finish(const TensorPtrs& t, int64_t first, Raw& r, const Hyper& h, const float* lut) {
+        momentum_finish<DT, ECCB, QUANT, KIND, FAST>(t, first, r, h, lut);
     }
 };
 

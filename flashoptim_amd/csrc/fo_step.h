@@ -2,11 +2,14 @@
 // requantisation helpers, the two grid shapes (single tensor by value / chunk table over many tensors) and
 // the host-side launch + dispatch templates.
 //
-// Work decomposition.  The unit of scheduling is a tile of 4096 consecutive elements of one tensor; a block
-// (FO_BLOCK_THREADS threads) walks the tiles of its chunk, each wavefront taking sub-tiles of 64 x EPL
-// elements (EPL = 8 for bf16/fp16, 4 for fp32; see fo_device.h for the access shape).  A quantisation group is
-// 32/EPL neighbouring lanes, so the group absmax is in-register maxes plus two or three DPP moves.  LDS only
-// holds the table that turns a first-moment code byte into its dequantised value.
+// Work decomposition.  A wavefront processes sub-tiles of 64 x EPL consecutive elements (EPL = 8 for bf16/fp16,
+// 4 for fp32; see fo_device.h for the access shape); a workgroup of FO_BLOCK_THREADS threads covers
+// FO_BLOCK_THREADS/64 x FO_SUBTILES_PER_WAVE neighbouring sub-tiles (its "span") and retires.  Workgroups are
+// deliberately tiny and short-lived: streaming from HBM is measurably better with many one-wavefront workgroups
+// that each touch every stream once than with larger or persistent ones.  The multi-tensor grid addresses work
+// through a chunk table in units of 4096-element tiles; a tile is an integer number of spans.  A quantisation
+// group is 32/EPL neighbouring lanes, so the group absmax is in-register maxes plus two or three DPP moves.
+// LDS only holds the table that turns a first-moment code byte into its dequantised value.
 //
 // "ref:" cites /root/reference/flashoptim/optimizers.py.
 #pragma once
@@ -16,7 +19,10 @@
 #include "../../include/flashoptim_hip.h"
 
 #ifndef FO_BLOCK_THREADS
-#define FO_BLOCK_THREADS 512
+#define FO_BLOCK_THREADS 64
+#endif
+#ifndef FO_SUBTILES_PER_WAVE
+#define FO_SUBTILES_PER_WAVE 1
 #endif
 #ifndef FO_LUT_REPL
 #define FO_LUT_REPL 1
@@ -26,7 +32,8 @@ namespace fo {
 
 constexpr int kBlockThreads = FO_BLOCK_THREADS;
 constexpr int kBlockWaves = kBlockThreads / 64;
-using StepLut = Lut<FO_LUT_REPL>;
+constexpr int kPerWave = FO_SUBTILES_PER_WAVE;
+using StepLut = Lut<FO_LUT_REPL, kBlockThreads>;
 
 struct TensorPtrs {
     void* param;
@@ -64,8 +71,12 @@ __device__ __forceinline__ void read_master(float (&p)[EPL], const Pack<DTypeInf
 #pragma unroll
     for (int k = 0; k < EPL; ++k) {
         const float w = widen<DT, EPL>(praw, k);
+#ifdef FO_EXPERIMENT_LIGHT
+        p[k] = w + ecc_to_float<ECCB, EPL>(eraw, k);
+#else
         if constexpr (ECCB > 0) p[k] = ecc_join<DT, ECCB>(w, ecc_to_float<ECCB, EPL>(eraw, k));
         else p[k] = w;
+#endif
     }
 }
 
@@ -78,10 +89,14 @@ __device__ __forceinline__ void write_master(const float (&p)[EPL], Pack<DTypeIn
     for (int k = 0; k < EPL; k += 2) {
         float wa, wb;
         narrow_pair<DT, EPL>(pout, k, p[k], p[k + 1], wa, wb);
+#ifdef FO_EXPERIMENT_LIGHT
+        eb[k] = as_u32(p[k] - wa); eb[k + 1] = as_u32(p[k + 1] - wb);
+#else
         if constexpr (ECCB > 0) {
             eb[k] = ecc_split_bits<DT, ECCB, false>(p[k], wa);
             eb[k + 1] = ecc_split_bits<DT, ECCB, false>(p[k + 1], wb);
         }
+#endif
     }
     if constexpr (ECCB > 0) pack_codes<ECCB, EPL>(eb, eout);
 }
@@ -100,10 +115,11 @@ __device__ __forceinline__ void quantize_mom(const float (&m)[EPL], float am, Pa
     pack_codes<1, EPL>(b, out);
 }
 
-// Quantises sqrt(v): code = rne(255 * r / av) with 255/av formed once per lane (ref:2408-2419).
+// Quantises sqrt(v): code = rne(255 * r / av) with 255/av formed once per lane from the hardware reciprocal
+// (ref:2408-2419; av >= 1e-12, so the reciprocal is a normal number).
 template <int EPL>
 __device__ __forceinline__ void quantize_var(const float (&r)[EPL], float av, Pack<1, EPL>& out) {
-    const float scale = div_rn(255.0f, av);
+    const float scale = 255.0f * __builtin_amdgcn_rcpf(av);
     u32 b[EPL];
 #pragma unroll
     for (int k = 0; k < EPL; ++k) b[k] = as_u32(fmaf(r[k], scale, kMagic));
@@ -123,48 +139,84 @@ __device__ __forceinline__ void narrow_all(const float (&x)[EPL], Pack<DTypeInfo
 // kernels
 // ------------------------------------------------------------------------------------------------
 
-// One tile: every wavefront of the block takes sub-tiles wave, wave + W, ... of the tile.
-template <class Op>
-__device__ __forceinline__ void run_tile(const TensorPtrs& t, int64_t tile, bool aligned, const typename Op::Hyper& h,
-                                         const float* lut_lane) {
-    constexpr int kSub = 64 * Op::kEpl;              // elements per sub-tile
-    constexpr int kSubsPerTile = kTileElems / kSub;  // 8 (EPL 8) or 16 (EPL 4)
-    const int64_t tile_base = tile * (int64_t)kTileElems;
+// Elements one workgroup covers.
+template <class Op> struct Span {
+    static constexpr int kSub = 64 * Op::kEpl;                       // elements per sub-tile
+    static constexpr int kElems = kBlockWaves * kPerWave * kSub;     // elements per workgroup
+    static constexpr int kPerTile = kTileElems / kElems;             // workgroups per 4096-element tile
+    static_assert(kElems <= kTileElems && kTileElems % kElems == 0, "a tile must be a whole number of workgroup spans");
+};
+
+// One span starting at element `base` of tensor t.  All loads are issued first, `between()` runs while they are
+// in flight (the workgroup commits the LDS table there), then the sub-tiles are finished one after the other.
+template <class Op, class Between>
+__device__ __forceinline__ void run_span(const TensorPtrs& t, int64_t base, bool aligned, const typename Op::Hyper& h,
+                                         const float* lut_lane, Between&& between) {
+    constexpr int kSub = Span<Op>::kSub;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    // block-uniform choice: whole tile in range and every stream 16-byte aligned -> straight-line vector path
-    if (aligned && (tile_base + kTileElems <= t.n)) {
-        for (int s = wave; s < kSubsPerTile; s += kBlockWaves)
-            Op::template lane<true>(t, tile_base + s * kSub + lane * Op::kEpl, h, lut_lane);
+    // wavefront w takes sub-tiles w, w + W, ... of the span
+    const int64_t first0 = base + (int64_t)wave * kSub + lane * Op::kEpl;
+    constexpr int64_t kStride = (int64_t)kBlockWaves * kSub;
+    typename Op::Raw raw[kPerWave];
+    // workgroup-uniform choice of the access mode
+    if (aligned) {
+        if (base + Span<Op>::kElems <= t.n) {
+#pragma unroll
+            for (int i = 0; i < kPerWave; ++i) Op::template load<kVector>(t, first0 + i * kStride, raw[i]);
+            between();
+#pragma unroll
+            for (int i = 0; i < kPerWave; ++i) Op::template finish<kVector>(t, first0 + i * kStride, raw[i], h, lut_lane);
+        } else {
+#pragma unroll
+            for (int i = 0; i < kPerWave; ++i) Op::template load<kLane>(t, first0 + i * kStride, raw[i]);
+            between();
+#pragma unroll
+            for (int i = 0; i < kPerWave; ++i) Op::template finish<kLane>(t, first0 + i * kStride, raw[i], h, lut_lane);
+        }
     } else {
-        for (int s = wave; s < kSubsPerTile; s += kBlockWaves)
-            Op::template lane<false>(t, tile_base + s * kSub + lane * Op::kEpl, h, lut_lane);
+        between();
+#pragma unroll 1
+        for (int i = 0; i < kPerWave; ++i) {
+            Op::template load<kGuarded>(t, first0 + i * kStride, raw[0]);
+            Op::template finish<kGuarded>(t, first0 + i * kStride, raw[0], h, lut_lane);
+        }
     }
 }
 
-template <class Op>
-__global__ __launch_bounds__(kBlockThreads) void step_single_kernel(TensorPtrs t, typename Op::Hyper h, int tiles_per_block) {
-    __shared__ float lut[Op::kNeedsLut ? StepLut::kFloats : 1];
-    if constexpr (Op::kNeedsLut) StepLut::build(lut);
-    const float* lut_lane = StepLut::lane_base(lut);
-    const bool aligned = all_aligned16(t);
-    const int64_t n_tiles = (t.n + kTileElems - 1) / kTileElems;
-    const int64_t t0 = (int64_t)blockIdx.x * tiles_per_block;
-    const int64_t t1 = t0 + tiles_per_block < n_tiles ? t0 + tiles_per_block : n_tiles;
-    for (int64_t tile = t0; tile < t1; ++tile) run_tile<Op>(t, tile, aligned, h, lut_lane);
-}
+// Commits the first-moment table to LDS once per workgroup, at the first call.
+template <bool NEEDED> struct LutCommit {
+    float* lut; StepLut::Frag frag; bool done;
+    __device__ __forceinline__ void operator()() {
+        if constexpr (NEEDED) {
+            if (!done) { StepLut::commit(lut, frag); done = true; }
+        }
+    }
+};
 
 template <class Op>
+__global__ __launch_bounds__(kBlockThreads) void step_single_kernel(TensorPtrs t, typename Op::Hyper h) {
+    __shared__ __align__(16) float lut[Op::kNeedsLut ? StepLut::kFloats : 4];
+    LutCommit<Op::kNeedsLut> commit{lut, {}, false};
+    if constexpr (Op::kNeedsLut) commit.frag = StepLut::fetch();
+    run_span<Op>(t, (int64_t)blockIdx.x * Span<Op>::kElems, all_aligned16(t), h, StepLut::lane_base(lut), commit);
+}
+
+// Workgroup b works on chunk b / kPerTile and takes span b % kPerTile of each of the chunk's tiles.
+template <class Op>
 __global__ __launch_bounds__(kBlockThreads) void step_multi_kernel(const fo_tensor_desc* __restrict__ descs,
-                                                                   const fo_chunk* __restrict__ chunks, int64_t n_chunks,
-                                                                   typename Op::Hyper h) {
-    __shared__ float lut[Op::kNeedsLut ? StepLut::kFloats : 1];
-    if constexpr (Op::kNeedsLut) StepLut::build(lut);
+                                                                   const fo_chunk* __restrict__ chunks, typename Op::Hyper h) {
+    __shared__ __align__(16) float lut[Op::kNeedsLut ? StepLut::kFloats : 4];
+    constexpr int kPerTile = Span<Op>::kPerTile;
+    const fo_chunk ck = chunks[blockIdx.x / kPerTile];
+    const TensorPtrs t = load_desc(descs + ck.tensor);
+    LutCommit<Op::kNeedsLut> commit{lut, {}, false};
+    if constexpr (Op::kNeedsLut) commit.frag = StepLut::fetch();
     const float* lut_lane = StepLut::lane_base(lut);
-    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const fo_chunk ck = chunks[c];
-        const TensorPtrs t = load_desc(descs + ck.tensor);
-        const bool aligned = all_aligned16(t);
-        for (int i = 0; i < ck.n_tiles; ++i) run_tile<Op>(t, (int64_t)ck.first_tile + i, aligned, h, lut_lane);
+    const bool aligned = all_aligned16(t);
+    const int64_t in_tile = (int64_t)(blockIdx.x % kPerTile) * Span<Op>::kElems;
+    for (int i = 0; i < ck.n_tiles; ++i) {
+        const int64_t base = ((int64_t)ck.first_tile + i) * kTileElems + in_tile;
+        if (base < t.n) run_span<Op>(t, base, aligned, h, lut_lane, commit);
     }
 }
 
@@ -213,22 +265,32 @@ inline int validate_multi(const fo_tensor_desc* descs, int64_t n_tensors, const 
 }
 
 
+// Streaming from HBM degrades when a compute unit keeps too many bytes in flight, and a step wavefront has
+// several KiB of loads outstanding.  Each kernel family therefore names how many workgroups it wants resident
+// per compute unit (Op::kResidentWorkgroups) and the launch requests enough unused LDS (160 KiB per compute
+// unit) to enforce it.
+template <class Op> inline unsigned lds_pad_bytes() {
+    const int env = step_lds_pad_bytes();
+    if (env >= 0) return (unsigned)env;
+    constexpr int kStatic = Op::kNeedsLut ? fo::StepLut::kFloats * 4 : 16;
+    constexpr int kTotal = (160 * 1024 / Op::kResidentWorkgroups) & ~255;
+    return kTotal > kStatic ? kTotal - kStatic : 0;
+}
+
 template <class Op>
 int launch_single(const fo::TensorPtrs& t, const typename Op::Hyper& h, hipStream_t stream) {
-    // One pass over the tensor with many short-lived blocks: the hardware scheduler keeps neighbouring tiles
-    // in flight together, which streams from HBM measurably better than a persistent grid-stride loop.
-    const int64_t n_tiles = (t.n + fo::kTileElems - 1) / fo::kTileElems;
-    const int tpb = tiles_per_block();
-    const int64_t grid = (n_tiles + tpb - 1) / tpb;
-    if (grid > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "tensor too large for one launch");
-    hipLaunchKernelGGL(fo::step_single_kernel<Op>, dim3((unsigned)grid), dim3(fo::kBlockThreads), 0, stream, t, h, tpb);
+    // one pass over the tensor, one short-lived workgroup per span
+    const int64_t grid = (t.n + fo::Span<Op>::kElems - 1) / fo::Span<Op>::kElems;
+    if (grid > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "tensor too large for one launch (%lld elements)", (long long)t.n);
+    hipLaunchKernelGGL(fo::step_single_kernel<Op>, dim3((unsigned)grid), dim3(fo::kBlockThreads), lds_pad_bytes<Op>(), stream, t, h);
     return check_hip(hipGetLastError(), "step kernel launch");
 }
 
 template <class Op>
 int launch_multi(const fo_tensor_desc* descs, const fo_chunk* chunks, int64_t n_chunks, const typename Op::Hyper& h, hipStream_t stream) {
-    const int64_t grid = n_chunks < INT32_MAX ? n_chunks : INT32_MAX;  // one chunk per block; the loop covers the rest
-    hipLaunchKernelGGL(fo::step_multi_kernel<Op>, dim3((unsigned)grid), dim3(fo::kBlockThreads), 0, stream, descs, chunks, n_chunks, h);
+    const int64_t grid = n_chunks * fo::Span<Op>::kPerTile;
+    if (grid > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "chunk table too large for one launch (%lld chunks)", (long long)n_chunks);
+    hipLaunchKernelGGL(fo::step_multi_kernel<Op>, dim3((unsigned)grid), dim3(fo::kBlockThreads), lds_pad_bytes<Op>(), stream, descs, chunks, h);
     return check_hip(hipGetLastError(), "multi-tensor step kernel launch");
 }
 

@@ -86,7 +86,7 @@ typedef struct fo_tensor_desc {
     void *param;
     const void *grad;
     void *ecc;        /* NULL when ecc_bytes == 0 */
-    void *mom;        /* NULL for fo_multi_sgd_plain_step */
+    void *mom;        /* first-moment state (codes or plain values) */
     void *mom_scales; /* NULL when not quantized */
     void *var;        /* Adam only */
     void *var_scales; /* Adam only, NULL when not quantized */
@@ -100,7 +100,9 @@ typedef struct fo_chunk {
     int32_t reserved;
 } fo_chunk;
 
+#ifndef FO_TILE_ELEMS
 #define FO_TILE_ELEMS 4096
+#endif
 
 /* Host helper: number of chunks fo_build_chunks will emit for these tensor lengths (0-length tensors emit
  * none).  tiles_per_chunk <= 0 selects the library default. */
