@@ -235,7 +235,7 @@ def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="llama8b-mwb24")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()

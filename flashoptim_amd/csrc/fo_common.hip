@@ -10,11 +10,15 @@
 
 namespace fo {
 
-constexpr int kCopyThreads = 256;
+constexpr int kCopyThreads = 64;
 
-// plain copy with the same access shape; calibrates byte counters and shows the attainable streaming rate
-__global__ __launch_bounds__(kCopyThreads) void copy_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, int64_t n_vec) {
-    for (int64_t i = (int64_t)blockIdx.x * kCopyThreads + threadIdx.x; i < n_vec; i += (int64_t)gridDim.x * kCopyThreads)
+// Plain copy in the step kernels' geometry (one-wavefront workgroups, one 128-bit non-temporal load and store per
+// lane, each workgroup retires after 1 KiB): calibrates byte counters and shows the attainable streaming rate.
+// Every workgroup makes `passes` such accesses, `stride_vec` vectors apart (1 for ordinary sizes).
+__global__ __launch_bounds__(kCopyThreads) void copy_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, int64_t n_vec,
+                                                            int64_t stride_vec, int passes) {
+    int64_t i = (int64_t)blockIdx.x * kCopyThreads + threadIdx.x;
+    for (int k = 0; k < passes && i < n_vec; ++k, i += stride_vec)
         __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
@@ -126,13 +130,13 @@ int fo_copy_bytes(void* dst, const void* src, int64_t n_bytes, void* stream) {
     if (n_bytes < 0 || (n_bytes & 15)) return fail(FO_ERR_INVALID_ARGUMENT, "n_bytes must be a non-negative multiple of 16");
     if (n_bytes == 0) return 0;
     if (!dst || !src || (((uintptr_t)dst | (uintptr_t)src) & 15)) return fail(FO_ERR_INVALID_ARGUMENT, "copy pointers must be 16-byte aligned");
-    const int cus = compute_units();
-    if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
     const int64_t n_vec = n_bytes / 16;
     const int64_t want = (n_vec + fo::kCopyThreads - 1) / fo::kCopyThreads;
-    const int64_t cap = (int64_t)cus * kBlocksPerCu * 2;
-    hipLaunchKernelGGL(fo::copy_kernel, dim3((unsigned)(want < cap ? want : cap)), dim3(fo::kCopyThreads), 0, (hipStream_t)stream,
-                       (fo::u32x4*)dst, (const fo::u32x4*)src, n_vec);
+    // one access per workgroup up to 2^31 - 1 workgroups (2 TiB); beyond that every workgroup makes several passes
+    const int passes = (int)((want + INT32_MAX - 1) / INT32_MAX);
+    const int64_t grid = (want + passes - 1) / passes;
+    hipLaunchKernelGGL(fo::copy_kernel, dim3((unsigned)grid), dim3(fo::kCopyThreads), 0, (hipStream_t)stream,
+                       (fo::u32x4*)dst, (const fo::u32x4*)src, n_vec, grid * fo::kCopyThreads, passes);
     return check_hip(hipGetLastError(), "copy kernel launch");
 }
 

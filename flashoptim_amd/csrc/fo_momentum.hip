@@ -112,7 +112,7 @@ __device__ __forceinline__ void momentum_finish(const TensorPtrs& t, int64_t fir
 template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumOp {
     using Hyper = MomentumHyper;
     static constexpr bool kNeedsLut = QUANT && KIND != KIND_PLAIN;
-    static constexpr int kResidentWorkgroups = 20;  // measured optimum on MI355X (3 KiB of loads per wavefront)
+    static constexpr int kLdsBytes = 7936;  // 20 resident workgroups: measured optimum on MI355X (3 KiB of loads per wavefront)
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = MomentumRaw<DT, ECCB, QUANT, KIND>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, int64_t first, Raw& r) {

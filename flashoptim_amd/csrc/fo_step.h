@@ -71,12 +71,8 @@ __device__ __forceinline__ void read_master(float (&p)[EPL], const Pack<DTypeInf
 #pragma unroll
     for (int k = 0; k < EPL; ++k) {
         const float w = widen<DT, EPL>(praw, k);
-#ifdef FO_EXPERIMENT_LIGHT
-        p[k] = w + ecc_to_float<ECCB, EPL>(eraw, k);
-#else
         if constexpr (ECCB > 0) p[k] = ecc_join<DT, ECCB>(w, ecc_to_float<ECCB, EPL>(eraw, k));
         else p[k] = w;
-#endif
     }
 }
 
@@ -89,14 +85,10 @@ __device__ __forceinline__ void write_master(const float (&p)[EPL], Pack<DTypeIn
     for (int k = 0; k < EPL; k += 2) {
         float wa, wb;
         narrow_pair<DT, EPL>(pout, k, p[k], p[k + 1], wa, wb);
-#ifdef FO_EXPERIMENT_LIGHT
-        eb[k] = as_u32(p[k] - wa); eb[k + 1] = as_u32(p[k + 1] - wb);
-#else
         if constexpr (ECCB > 0) {
             eb[k] = ecc_split_bits<DT, ECCB, false>(p[k], wa);
             eb[k + 1] = ecc_split_bits<DT, ECCB, false>(p[k + 1], wb);
         }
-#endif
     }
     if constexpr (ECCB > 0) pack_codes<ECCB, EPL>(eb, eout);
 }
@@ -147,6 +139,13 @@ template <class Op> struct Span {
     static_assert(kElems <= kTileElems && kTileElems % kElems == 0, "a tile must be a whole number of workgroup spans");
 };
 
+// Order of the spans.  The hardware deals workgroups round-robin to the 8 XCDs (workgroup b runs on XCD b % 8),
+// each with its own L2, so with the identity order used here the 8 XCDs sweep the tensor together, 1 KiB of
+// parameters each.  A 128-byte line of fp16 group scales (2048 elements) is then read through four L2s:
+// rocprofv3's FETCH_SIZE shows the scale reads four times over (+0.375 B per element).  Giving each XCD runs of
+// four consecutive spans removes that over-fetch exactly but streams 5 % slower (4 KiB per XCD instead of
+// 1 KiB), so the identity order stays.
+
 // One span starting at element `base` of tensor t.  All loads are issued first, `between()` runs while they are
 // in flight (the workgroup commits the LDS table there), then the sub-tiles are finished one after the other.
 template <class Op, class Between>
@@ -196,9 +195,10 @@ template <bool NEEDED> struct LutCommit {
 template <class Op>
 __global__ __launch_bounds__(kBlockThreads) void step_single_kernel(TensorPtrs t, typename Op::Hyper h) {
     __shared__ __align__(16) float lut[Op::kNeedsLut ? StepLut::kFloats : 4];
+    const int64_t base = (int64_t)blockIdx.x * Span<Op>::kElems;
     LutCommit<Op::kNeedsLut> commit{lut, {}, false};
     if constexpr (Op::kNeedsLut) commit.frag = StepLut::fetch();
-    run_span<Op>(t, (int64_t)blockIdx.x * Span<Op>::kElems, all_aligned16(t), h, StepLut::lane_base(lut), commit);
+    run_span<Op>(t, base, all_aligned16(t), h, StepLut::lane_base(lut), commit);
 }
 
 // Workgroup b works on chunk b / kPerTile and takes span b % kPerTile of each of the chunk's tiles.
@@ -207,13 +207,14 @@ __global__ __launch_bounds__(kBlockThreads) void step_multi_kernel(const fo_tens
                                                                    const fo_chunk* __restrict__ chunks, typename Op::Hyper h) {
     __shared__ __align__(16) float lut[Op::kNeedsLut ? StepLut::kFloats : 4];
     constexpr int kPerTile = Span<Op>::kPerTile;
-    const fo_chunk ck = chunks[blockIdx.x / kPerTile];
+    const unsigned b = blockIdx.x;
+    const fo_chunk ck = chunks[b / kPerTile];
     const TensorPtrs t = load_desc(descs + ck.tensor);
     LutCommit<Op::kNeedsLut> commit{lut, {}, false};
     if constexpr (Op::kNeedsLut) commit.frag = StepLut::fetch();
     const float* lut_lane = StepLut::lane_base(lut);
     const bool aligned = all_aligned16(t);
-    const int64_t in_tile = (int64_t)(blockIdx.x % kPerTile) * Span<Op>::kElems;
+    const int64_t in_tile = (int64_t)(b % kPerTile) * Span<Op>::kElems;
     for (int i = 0; i < ck.n_tiles; ++i) {
         const int64_t base = ((int64_t)ck.first_tile + i) * kTileElems + in_tile;
         if (base < t.n) run_span<Op>(t, base, aligned, h, lut_lane, commit);
@@ -266,15 +267,15 @@ inline int validate_multi(const fo_tensor_desc* descs, int64_t n_tensors, const 
 
 
 // Streaming from HBM degrades when a compute unit keeps too many bytes in flight, and a step wavefront has
-// several KiB of loads outstanding.  Each kernel family therefore names how many workgroups it wants resident
-// per compute unit (Op::kResidentWorkgroups) and the launch requests enough unused LDS (160 KiB per compute
-// unit) to enforce it.
+// several KiB of loads outstanding.  Each kernel family therefore names the LDS footprint it wants per
+// workgroup (Op::kLdsBytes; a compute unit has 160 KiB, so 11008 bytes admit 14 workgroups) and the launch
+// requests the difference to the kernel's own table as unused dynamic LDS.  The values sit in the middle of the
+// measured plateaus, away from the residencies (13 and 16 for Adam) where throughput drops by 4-5 %.
 template <class Op> inline unsigned lds_pad_bytes() {
     const int env = step_lds_pad_bytes();
     if (env >= 0) return (unsigned)env;
     constexpr int kStatic = Op::kNeedsLut ? fo::StepLut::kFloats * 4 : 16;
-    constexpr int kTotal = (160 * 1024 / Op::kResidentWorkgroups) & ~255;
-    return kTotal > kStatic ? kTotal - kStatic : 0;
+    return Op::kLdsBytes > kStatic ? Op::kLdsBytes - kStatic : 0;
 }
 
 template <class Op>
