@@ -69,7 +69,7 @@ class _Bucket:
     quantized: bool
     params: list                      # the nn.Parameters, in table order
     tensors: list                     # StepTensors with grad=None (state tensors only)
-    plan: Optional[BucketPlan]        # multi-tensor tables; None for single-tensor / momentum-free buckets
+    plan: Optional[BucketPlan]        # multi-tensor tables; None for single-tensor buckets
     step_tensors: list                # the CPU `step` scalars of the bucket (Adam), else empty
     step_value: Optional[int]
 
@@ -80,6 +80,8 @@ class _GroupCache:
     params: list
     signature: Any
     buckets: list
+    # check_numerics: log2 of the coarsest weight resolution over the group's parameters (None: nothing to check)
+    numerics_needed: Optional[float] = None
 
 
 class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
@@ -228,16 +230,26 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         return tensor.to_local() if hasattr(tensor, "to_local") else tensor
 
     # ------------------------------------------------------------------------------------- numerics check
+    def _recompute_stats(self, params: list) -> None:
+        """Largest magnitude of every given parameter: one launch per (device, dtype) and one synchronisation per
+        device, instead of the reference's ``abs().max().item()`` per tensor (ref:656-673)."""
+        tensors = [self._get_tensor_for_stats(p).detach() for p in params]
+        for p, maxabs in zip(params, kernels.absmax_many(tensors)):
+            self._transient_state.setdefault(id(p), {})["maxabs"] = maxabs
+        self._plan_epoch += 1  # cached numerics verdicts are stale
+
     def _recompute_stats_for_param(self, p: torch.Tensor) -> None:
-        t = self._get_tensor_for_stats(p)
-        maxabs = float(t.detach().abs().max().item()) if t.numel() else 0
-        self._transient_state.setdefault(id(p), {})["maxabs"] = maxabs
+        self._recompute_stats([p])
 
     def recompute_param_stats(self) -> None:
         """Refresh the cached largest magnitude of every parameter (used by ``check_numerics``)."""
-        for group in self.param_groups:
-            for p in group["params"]:
-                self._recompute_stats_for_param(p)
+        self._recompute_stats([p for group in self.param_groups for p in group["params"]])
+
+    def _numerics_needed(self, p: torch.Tensor, master_bytewidth: int) -> Optional[float]:
+        maxabs = self._transient_state.get(id(p), {}).get("maxabs", 0)
+        if maxabs <= 0 or not math.isfinite(maxabs):
+            return None
+        return _log2_min_expressible_step_size(dtype=p.dtype, maxabs=maxabs, master_bytewidth=master_bytewidth)
 
     def _check_param_numerics(self, p: torch.Tensor, lr: float, master_bytewidth: int) -> None:
         if lr == 0.0:
@@ -371,7 +383,12 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         """Full per-parameter planning (state creation, checks, counters), then one launch per bucket; leaves a
         cache behind when every parameter of the group took part."""
         planned: dict[LaunchKey, list] = {}
-        complete = not self._check_numerics
+        complete = True
+        if self._check_numerics:  # one scan for every parameter that has no cached statistic yet
+            missing = [p for p in group["params"]
+                       if p.grad is not None and self._transient_state.get(id(p), {}).get("maxabs") is None]
+            if missing:
+                self._recompute_stats(missing)
         for p in group["params"]:
             plan = self._plan_param(p, group)
             if plan is None:
@@ -386,7 +403,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
             tensors = [t for _, t in items]
             scalars = dict(key.scalars)
             plan = None
-            if key.kind != "plain" and len(tensors) > 1:
+            if len(tensors) > 1:
                 plan = BucketPlan(key.kind, key.dtype, key.ecc_bytes, key.quantized, tensors)
                 plan.launch(**scalars)
             else:
@@ -398,8 +415,12 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
             buckets.append(_Bucket(key.kind, key.dtype, key.ecc_bytes, key.quantized, [p for p, _ in items], tensors,
                                    plan, step_tensors, scalars.get("step")))
         if complete and buckets:
+            needed = None
+            if self._check_numerics:
+                each = [self._numerics_needed(p, group["master_bytewidth"]) for p in group["params"]]
+                needed = max((x for x in each if x is not None), default=None)
             self._group_cache[index] = _GroupCache(self._plan_epoch, list(group["params"]),
-                                                   self._plan_signature(group), buckets)
+                                                   self._plan_signature(group), buckets, needed)
         else:
             self._group_cache.pop(index, None)
 
@@ -438,6 +459,13 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
                     t.grad = None
         return True
 
+    def _cached_numerics_ok(self, cache: _GroupCache, group: dict[str, Any]) -> bool:
+        """check_numerics for a cached group: the weights' resolution is cached, only lr can have moved.  False
+        sends the group through the full path, which raises the NumericsError naming the parameter."""
+        if not self._check_numerics or cache.numerics_needed is None or group["lr"] == 0.0:
+            return True
+        return cache.numerics_needed <= math.log2(group["lr"] * self._min_step_size_relative_to_lr())
+
     @torch.no_grad()
     def step(self, closure: Optional[Callable] = None) -> Optional[torch.Tensor]:
         if self._gradient_release:
@@ -456,7 +484,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
             if (
                 cache is not None
                 and cache.epoch == self._plan_epoch
-                and not self._check_numerics
+                and self._cached_numerics_ok(cache, group)
                 and len(cache.params) == len(group["params"])
                 and all(a is b for a, b in zip(cache.params, group["params"]))
                 and cache.signature == self._plan_signature(group)

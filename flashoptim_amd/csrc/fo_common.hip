@@ -65,6 +65,13 @@ int default_tiles_per_chunk() {
     return value;
 }
 
+int validate_multi_tables(const void* descs, int64_t n_tensors, const void* chunks, int64_t n_chunks, int dtype) {
+    if (n_tensors < 0 || n_chunks < 0) return fail(FO_ERR_INVALID_ARGUMENT, "negative count");
+    if (dtype < FO_F32 || dtype > FO_F16) return fail(FO_ERR_INVALID_ARGUMENT, "unknown dtype %d", dtype);
+    if (n_chunks > 0 && (!descs || !chunks)) return fail(FO_ERR_INVALID_ARGUMENT, "descs/chunks must not be NULL");
+    return 0;
+}
+
 int compute_units() {
     static thread_local int cached_dev = -1, cached_cus = 0;
     int dev = 0;

@@ -175,4 +175,12 @@ int fo_multi_momentum_step(const fo_tensor_desc* descs, int64_t n_tensors, const
     return do_lion ? dispatch<LionOp>(dtype, ecc_bytes, quantized, L) : dispatch<SgdOp>(dtype, ecc_bytes, quantized, L);
 }
 
+int fo_multi_sgd_plain_step(const fo_tensor_desc* descs, int64_t n_tensors, const fo_chunk* chunks, int64_t n_chunks,
+                            int dtype, int ecc_bytes, float lr, float weight_decay, int decoupled, void* stream) {
+    if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
+    if (n_chunks == 0) return 0;
+    MultiLauncher<fo::MomentumHyper> L{descs, chunks, n_chunks, make_momentum_hyper(lr, 0.0f, 1.0f, weight_decay, decoupled, 0), (hipStream_t)stream};
+    return dispatch<PlainOp>(dtype, ecc_bytes, 0, L);
+}
+
 }  // extern "C"

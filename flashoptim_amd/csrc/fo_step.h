@@ -257,11 +257,9 @@ inline int validate_state(const void* state, const void* scales, int quantized, 
 
 inline int validate_multi(const fo_tensor_desc* descs, int64_t n_tensors, const fo_chunk* chunks, int64_t n_chunks,
                           int dtype, int ecc_bytes) {
-    if (n_tensors < 0 || n_chunks < 0) return fail(FO_ERR_INVALID_ARGUMENT, "negative count");
-    if (dtype < FO_F32 || dtype > FO_F16) return fail(FO_ERR_INVALID_ARGUMENT, "unknown dtype %d", dtype);
+    if (int rc = validate_multi_tables(descs, n_tensors, chunks, n_chunks, dtype)) return rc;
     if (ecc_bytes < 0 || ecc_bytes > 2) return fail(FO_ERR_INVALID_ARGUMENT, "ecc_bytes must be 0, 1 or 2 (got %d)", ecc_bytes);
     if (dtype == FO_F32 && ecc_bytes != 0) return fail(FO_ERR_UNSUPPORTED, "fp32 parameters carry no ECC");
-    if (n_chunks > 0 && (!descs || !chunks)) return fail(FO_ERR_INVALID_ARGUMENT, "descs/chunks must not be NULL");
     return 0;
 }
 

@@ -296,6 +296,13 @@ def _sgd_plain_step(
     _native.check(rc, "fo_sgd_plain_step")
 
 
+def absmax_many(tensors) -> list:
+    """Largest magnitude of every tensor with one launch per (device, dtype); see ``launcher.absmax_many``."""
+    from .launcher import absmax_many as _impl
+
+    return _impl(tensors)
+
+
 def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
     """Device copy with the step kernels' access shape; a measurement aid (counter calibration, attainable
     streaming rate)."""

@@ -42,12 +42,61 @@ class StepTensors:
     var_scales: Optional[torch.Tensor] = None
 
 
+def chunk_table(numels: Sequence[int], tiles_per_chunk: int = 0) -> tuple[torch.Tensor, int]:
+    """The ``fo_chunk`` table for tensors of these lengths as a host byte tensor, and its entry count."""
+    lib = _native.lib()
+    n_tensors = len(numels)
+    lens = (ctypes.c_int64 * max(n_tensors, 1))(*numels)
+    n_chunks = lib.fo_count_chunks(lens, n_tensors, tiles_per_chunk)
+    if n_chunks < 0:
+        _native.check(int(n_chunks), "fo_count_chunks")
+    table = (FoChunk * max(n_chunks, 1))()
+    built = lib.fo_build_chunks(lens, n_tensors, tiles_per_chunk, table, n_chunks)
+    if built != n_chunks:
+        _native.check(int(built) if built < 0 else -1, "fo_build_chunks")
+    host = torch.frombuffer(bytearray(bytes(table)), dtype=torch.uint8)[: int(n_chunks) * ctypes.sizeof(FoChunk)]
+    return host, int(n_chunks)
+
+
+def absmax_many(tensors: Sequence[torch.Tensor]) -> list[float]:
+    """``float(t.abs().max())`` of every tensor (0 for empty ones): one launch per (device, dtype) and one
+    device-to-host copy per device, where the reference synchronises once per tensor
+    (``/root/reference/flashoptim/optimizers.py:656-673``).  A tensor holding a NaN reports NaN."""
+    out: list[float] = [0.0] * len(tensors)
+    groups: dict = {}
+    for i, t in enumerate(tensors):
+        if t.numel() == 0:
+            continue
+        if not t.is_cuda or t.dtype not in DTYPE_CODE or not t.is_contiguous():
+            out[i] = float(t.abs().max().item())  # dtypes and layouts the step kernels do not take either
+            continue
+        groups.setdefault((t.device, t.dtype), []).append(i)
+    pending = []
+    for (device, dtype), idx in groups.items():
+        table = (FoTensorDesc * len(idx))()
+        for d, i in zip(table, idx):
+            d.param, d.n = tensors[i].data_ptr(), tensors[i].numel()
+        chunks_host, n_chunks = chunk_table([tensors[i].numel() for i in idx], tiles_per_chunk=16)
+        with torch.cuda.device(device):
+            descs = torch.frombuffer(bytearray(bytes(table)), dtype=torch.uint8).to(device)
+            chunks = chunks_host.to(device)
+            result = torch.zeros(len(idx), dtype=torch.float32, device=device)
+            rc = _native.lib().fo_multi_absmax(descs.data_ptr(), len(idx), chunks.data_ptr(), n_chunks, DTYPE_CODE[dtype],
+                                               result.data_ptr(), _native.current_stream_ptr(device))
+        _native.check(rc, "fo_multi_absmax")
+        pending.append((idx, result, descs, chunks))
+    for idx, result, _descs, _chunks in pending:  # the tables stay alive until the results are read
+        for i, v in zip(idx, result.tolist()):
+            out[i] = float(v)
+    return out
+
+
 class BucketPlan:
     """Launch tables of one bucket: tensors that share kernel kind, dtype, ECC width and quantisation."""
 
     def __init__(self, kind: str, dtype: torch.dtype, ecc_bytes: int, quantized: bool,
                  tensors: Sequence[StepTensors], tiles_per_chunk: int = 0):
-        if kind not in ("adam", "momentum"):
+        if kind not in ("adam", "momentum", "plain"):
             raise ValueError(f"no multi-tensor kernel for kind {kind!r}")
         self.kind, self.dtype, self.ecc_bytes, self.quantized = kind, dtype, int(ecc_bytes), bool(quantized)
         self.device = tensors[0].param.device
@@ -64,17 +113,7 @@ class BucketPlan:
         self._keepalive = [(t.param, t.ecc, t.mom, t.mom_scales, t.var, t.var_scales) for t in tensors]
         self.grad_ptrs = [d.grad for d in self.table]
 
-        lib = _native.lib()
-        lens = (ctypes.c_int64 * self.n_tensors)(*numels)
-        n_chunks = lib.fo_count_chunks(lens, self.n_tensors, tiles_per_chunk)
-        if n_chunks < 0:
-            _native.check(int(n_chunks), "fo_count_chunks")
-        chunk_table = (FoChunk * max(n_chunks, 1))()
-        built = lib.fo_build_chunks(lens, self.n_tensors, tiles_per_chunk, chunk_table, n_chunks)
-        if built != n_chunks:
-            _native.check(int(built) if built < 0 else -1, "fo_build_chunks")
-        self.n_chunks = int(n_chunks)
-        host = torch.frombuffer(bytearray(bytes(chunk_table)), dtype=torch.uint8)[: self.n_chunks * ctypes.sizeof(FoChunk)]
+        host, self.n_chunks = chunk_table(numels, tiles_per_chunk)
         self.chunks_dev = host.to(self.device)
         self.descs_dev = torch.empty(self.n_tensors * ctypes.sizeof(FoTensorDesc), dtype=torch.uint8, device=self.device)
         self._dirty = True
@@ -106,8 +145,11 @@ class BucketPlan:
                 rc = lib.fo_multi_adam_step(*head, scalars["lr"], scalars["beta1"], scalars["beta2"], scalars["eps"],
                                             scalars["weight_decay"], int(scalars["decoupled"]), int(scalars["step"]),
                                             stream)
+            elif self.kind == "plain":
+                rc = lib.fo_multi_sgd_plain_step(*head[:6], scalars["lr"], scalars["weight_decay"],
+                                                 int(scalars["decoupled"]), stream)
             else:
                 rc = lib.fo_multi_momentum_step(*head, scalars["lr"], scalars["mom_coef"], scalars["update_coef"],
                                                 scalars["weight_decay"], int(scalars["decoupled"]),
                                                 int(scalars["nesterov"]), int(scalars["do_lion"]), stream)
-        _native.check(rc, f"fo_multi_{self.kind}_step")
+        _native.check(rc, "fo_multi_sgd_plain_step" if self.kind == "plain" else f"fo_multi_{self.kind}_step")

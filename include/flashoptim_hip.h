@@ -120,6 +120,21 @@ int fo_multi_momentum_step(const fo_tensor_desc *descs, int64_t n_tensors, const
                            float update_coef, float weight_decay, int decoupled, int nesterov, int do_lion,
                            void *stream);
 
+/* Momentum-free SGD over many tensors: the multi-tensor form of fo_sgd_plain_step (descs use param, grad, ecc, n). */
+int fo_multi_sgd_plain_step(const fo_tensor_desc *descs, int64_t n_tensors, const fo_chunk *chunks,
+                            int64_t n_chunks, int dtype, int ecc_bytes, float lr, float weight_decay,
+                            int decoupled, void *stream);
+
+/*
+ * Largest magnitude of every tensor of a list in one launch.  Replaces the per-tensor
+ * tensor.abs().max().item() behind check_numerics / recompute_param_stats (ref:656-673), which costs one device
+ * synchronisation per tensor.  descs use `param` (the data, `dtype` elements) and `n`; `out` is fp32[n_tensors],
+ * zeroed by the caller; out[i] receives max |x| of tensor i (NaN if it holds a NaN).  Chunks from
+ * fo_build_chunks with any tiles_per_chunk (larger chunks mean fewer atomic merges).
+ */
+int fo_multi_absmax(const fo_tensor_desc *descs, int64_t n_tensors, const fo_chunk *chunks, int64_t n_chunks,
+                    int dtype, float *out, void *stream);
+
 /*
  * Standalone group codec.  Replaces quantize / dequantize and their kernels (ref:2446-2538, 2541-2676).
  *   x            : `x_dtype` elements

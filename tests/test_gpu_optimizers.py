@@ -695,3 +695,85 @@ def test_cached_step_plan_follows_moving_missing_and_freed_gradients():
     del hold
     gc.collect()
     assert ref() is None, "the optimizer's cached plan kept a gradient alive"
+
+
+@pytest.mark.parametrize("dtype,mwb", [(torch.bfloat16, 24), (torch.bfloat16, 32), (torch.float32, None), (torch.float16, None)])
+@pytest.mark.parametrize("kwargs", [dict(weight_decay=0.0), dict(weight_decay=1e-2)])
+def test_momentum_free_sgd_multi_tensor_is_bit_identical_to_per_tensor_steps(dtype, mwb, kwargs):
+    """FlashSGD / FlashSGDW with momentum=0 (eager branch ref:1447-1465) as one multi-tensor launch."""
+    fo = _fo()
+    for factory in ("FlashSGD", "FlashSGDW"):
+        pa, pb = _make_params(_RAGGED, dtype, 2), _make_params(_RAGGED, dtype, 2)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            oa = getattr(fo, factory)(pa, lr=1e-2, momentum=0.0, master_weight_bits=mwb, **kwargs)
+            ob = getattr(fo, factory)(pb, lr=1e-2, momentum=0.0, master_weight_bits=mwb, **kwargs)
+        for it in range(3):
+            _set_grads(pa, 20 + it)
+            _set_grads(pb, 20 + it)
+            oa.step()
+            for p in pb:
+                ob.step_param(p)
+        for a, b in zip(pa, pb):
+            assert torch.equal(a, b)
+            assert "momentum_buffer" not in oa.state[a]
+            if mwb is not None:
+                assert torch.equal(oa.state[a]["error_bits"], ob.state[b]["error_bits"])
+
+
+def test_absmax_many_matches_torch():
+    from flashoptim_amd import kernels
+
+    g = torch.Generator().manual_seed(11)
+    tensors = []
+    for dtype in (torch.bfloat16, torch.float32, torch.float16):
+        for n in (1, 7, 31, 33, 511, 4096, 4097, 65536 + 5, 1_000_003):
+            tensors.append((torch.randn(n, generator=g) * 10 ** float(torch.randint(-3, 3, (1,), generator=g))).to(dtype).to(DEV))
+    tensors.append(torch.zeros(0, dtype=torch.bfloat16, device=DEV))
+    tensors.append(torch.zeros(100, dtype=torch.float32, device=DEV))
+    tensors.append(torch.randn(64, 64, generator=g).to(DEV).t())                       # non-contiguous
+    tensors.append(torch.randn(5000, generator=g, dtype=torch.float64).to(DEV))         # dtype without a kernel
+    big = torch.randn(3_000_000, generator=g).to(torch.bfloat16).to(DEV)
+    tensors.append(big[3:])                                                             # 2-byte aligned view
+    spike = torch.zeros(70000, dtype=torch.float16, device=DEV); spike[-1] = -60000.0
+    tensors.append(spike)
+    inf = torch.ones(5000, dtype=torch.float32, device=DEV); inf[123] = float("-inf")
+    tensors.append(inf)
+    got = kernels.absmax_many(tensors)
+    for t, v in zip(tensors, got):
+        want = float(t.abs().max().item()) if t.numel() else 0.0
+        assert v == want, (t.dtype, t.numel(), v, want)
+    nan = torch.ones(5000, dtype=torch.bfloat16, device=DEV); nan[4000] = float("nan")
+    import math
+    assert math.isnan(kernels.absmax_many([nan])[0])
+
+
+def test_check_numerics_with_cached_plans_and_one_scan():
+    """check_numerics keeps the cached step path: the weights' resolution is cached, a later drop of lr still
+    raises, and recompute_param_stats() refreshes the cached magnitudes (ref:656-673, 1149-1181)."""
+    fo = _fo()
+    params = _make_params([4096, 1000, 33], torch.bfloat16, 5)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        opt = fo.FlashLion(params, lr=1e-2, check_numerics=True, master_weight_bits=None)
+    initial = [float(p.detach().abs().max()) for p in params]
+    for it in range(3):
+        _set_grads(params, 30 + it)
+        opt.step()
+    assert opt._group_cache, "steps with check_numerics should leave a cached plan behind"
+    for p, want in zip(params, initial):  # scanned once, at the first step
+        assert opt._transient_state[id(p)]["maxabs"] == want
+    opt.param_groups[0]["lr"] = 1e-9
+    _set_grads(params, 40)
+    with pytest.raises(fo.NumericsError):
+        opt.step()
+    opt.param_groups[0]["lr"] = 1e-2
+    with torch.no_grad():
+        params[0].mul_(1e6)          # weights grow: the cached statistic is stale until recomputed
+    _set_grads(params, 41)
+    opt.step()
+    opt.recompute_param_stats()
+    assert opt._transient_state[id(params[0])]["maxabs"] == float(params[0].detach().abs().max())
+    _set_grads(params, 42)
+    with pytest.raises(fo.NumericsError):
+        opt.step()
