@@ -145,10 +145,12 @@ __global__ __launch_bounds__(kCodecThreads) void ecc_split_kernel(const float* x
 namespace {
 using namespace fo_host;
 
+// One short-lived workgroup per 4096-element tile (one pass streams better than a persistent grid here); the
+// kernels' tile loop only iterates for tensors beyond 2^31 - 1 tiles.
 unsigned grid_for(int64_t n, int cus) {
+    (void)cus;
     const int64_t tiles = (n + fo::kTileElems - 1) / fo::kTileElems;
-    const int64_t cap = (int64_t)cus * kBlocksPerCu;
-    return (unsigned)(tiles < cap ? tiles : cap);
+    return (unsigned)(tiles < INT32_MAX ? tiles : INT32_MAX);
 }
 
 }  // namespace
