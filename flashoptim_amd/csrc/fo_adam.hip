@@ -110,8 +110,8 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, int64_t first, 
         store_lane<1, EPL, FAST>(raw.m, t.mom, first, n);
         store_lane<1, EPL, FAST>(raw.v, t.var, first, n);
         if (live_group && (threadIdx.x & (32 / EPL - 1)) == 0) {                    // ref:2424-2434
-            t.mom_scales[group] = f32_to_f16_bits(am);
-            t.var_scales[group] = f32_to_f16_bits(av);
+            store_scale(t.mom_scales, group, f32_to_f16_bits(am));
+            store_scale(t.var_scales, group, f32_to_f16_bits(av));
         }
     } else {
         narrow_all<DT, EPL>(m, raw.m);                                              // ref:2435-2438

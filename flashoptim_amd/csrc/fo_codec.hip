@@ -44,7 +44,7 @@ __device__ __forceinline__ void quantize_lane(const void* x, void* codes, uint16
     Pack<1, EPL> out;
     pack_codes<1, EPL>(q, out);
     store_lane<1, EPL, FAST>(out, codes, first, n);
-    if ((FAST || first < n) && (threadIdx.x & (32 / EPL - 1)) == 0) scales[first >> 5] = f32_to_f16_bits(am);   // ref:2675-2676
+    if ((FAST || first < n) && (threadIdx.x & (32 / EPL - 1)) == 0) store_scale(scales, first >> 5, f32_to_f16_bits(am));   // ref:2675-2676
 }
 
 // ref:2541-2607 _triton_dequantize_kernel

@@ -78,19 +78,43 @@ __device__ __forceinline__ void load_vec(Pack<EB, EPL>& d, const void* base, int
         d.w[0] = __builtin_nontemporal_load(reinterpret_cast<const u32*>(p));
     }
 }
+// Stores carry the non-temporal hint and system-scope write-through (`sc0 sc1 nt`): a streamed line goes straight
+// to memory instead of sitting dirty in L2 until it is evicted, which measures 1.5 points of HBM peak better than
+// `nt` alone on MI355X.  The compiler has no builtin for this policy on plain global stores, hence the asm.
+// The hazard recogniser does not look inside asm: a store of more than 64 bits must be followed by two wait
+// states before a VALU instruction may overwrite its data registers, hence the `s_nop 1` after the 128-bit form.
+#ifndef FO_STORE_WRITE_THROUGH
+#define FO_STORE_WRITE_THROUGH 1
+#endif
 template <int EB, int EPL>
 __device__ __forceinline__ void store_vec(const Pack<EB, EPL>& d, void* base, int64_t first) {
     char* p = static_cast<char*>(base) + first * EB;
     if constexpr (Pack<EB, EPL>::kBytes == 16) {
         u32x4 v; v.x = d.w[0]; v.y = d.w[1]; v.z = d.w[2]; v.w = d.w[3];
+#if FO_STORE_WRITE_THROUGH
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+#else
         __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+#endif
     } else if constexpr (Pack<EB, EPL>::kBytes == 8) {
         u32x2 v; v.x = d.w[0]; v.y = d.w[1];
+#if FO_STORE_WRITE_THROUGH
+        asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1 nt" : : "v"(p), "v"(v) : "memory");
+#else
         __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
+#endif
     } else {
+#if FO_STORE_WRITE_THROUGH
+        asm volatile("global_store_dword %0, %1, off sc0 sc1 nt" : : "v"(p), "v"(d.w[0]) : "memory");
+#else
         __builtin_nontemporal_store(d.w[0], reinterpret_cast<u32*>(p));
+#endif
     }
 }
+
+// One fp16 group scale.  A wavefront writes 32 bytes of a 128-byte line here, so this store stays a cached
+// write-back store and lets L2 merge the pieces: written through like the streams it costs 3 points of HBM peak.
+__device__ __forceinline__ void store_scale(uint16_t* scales, int64_t group, uint16_t bits) { scales[group] = bits; }
 
 // Guarded path (tensor tails, unaligned views): element-wise accesses, out-of-range elements read as zero and
 // are never written (ref:1625-1630, 2296-2301 masked loads with other=0).

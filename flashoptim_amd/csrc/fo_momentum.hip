@@ -101,7 +101,7 @@ __device__ __forceinline__ void momentum_finish(const TensorPtrs& t, int64_t fir
             am = fmaxf(group_max<EPL>(am), 1e-12f);                                 // ref:1702-1703
             quantize_mom<EPL>(m, am, raw.m);
             store_lane<1, EPL, FAST>(raw.m, t.mom, first, n);
-            if (live_group && (threadIdx.x & (32 / EPL - 1)) == 0) t.mom_scales[group] = f32_to_f16_bits(am);  // ref:1713-1716
+            if (live_group && (threadIdx.x & (32 / EPL - 1)) == 0) store_scale(t.mom_scales, group, f32_to_f16_bits(am));  // ref:1713-1716
         } else {
             narrow_all<DT, EPL>(m, raw.m);                                          // ref:1717-1719
             store_lane<SB, EPL, FAST>(raw.m, t.mom, first, n);
