@@ -18,8 +18,11 @@ constexpr int kCopyThreads = 64;
 __global__ __launch_bounds__(kCopyThreads) void copy_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, int64_t n_vec,
                                                             int64_t stride_vec, int passes) {
     int64_t i = (int64_t)blockIdx.x * kCopyThreads + threadIdx.x;
-    for (int k = 0; k < passes && i < n_vec; ++k, i += stride_vec)
-        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+    for (int k = 0; k < passes && i < n_vec; ++k, i += stride_vec) {
+        Pack<4, 4> v;
+        load_vec<4, 4>(v, src, i * 4);
+        store_vec<4, 4>(v, dst, i * 4);
+    }
 }
 
 
