@@ -279,11 +279,12 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         quantize = hparams.get("quantize", self._quantize)
         for key, spec in self._quantized_state_spec().items():
             if key not in state:
-                state[key] = _MaybeQuantizedTensor(
-                    self._initial_value_for_state_var(local, key),
-                    try_quantize=quantize, signed=spec.signed, sqrt=spec.sqrt, softsign=spec.softsign,
-                    storage_dtype=local.dtype,
-                )
+                kw = dict(try_quantize=quantize, signed=spec.signed, sqrt=spec.sqrt, softsign=spec.softsign,
+                          storage_dtype=local.dtype)
+                if type(self)._initial_value_for_state_var is FlashOptimizer._initial_value_for_state_var:
+                    state[key] = _MaybeQuantizedTensor.zeros_like(local, **kw)  # zero start: nothing to quantise
+                else:
+                    state[key] = _MaybeQuantizedTensor(self._initial_value_for_state_var(local, key), **kw)
         extra_bytes = hparams["master_bytewidth"] - _DTYPE_WIDTHS[p.dtype]
         if extra_bytes > 0 and state.get("error_bits") is None:
             state["error_bits"] = torch.zeros_like(local, dtype=torch.int8 if extra_bytes == 1 else torch.int16)

@@ -122,6 +122,25 @@ class _MaybeQuantizedTensor:
             self._quantized = None
             self._scales = None
 
+    @classmethod
+    def zeros_like(cls, ref: torch.Tensor, try_quantize: bool = True, signed: bool = True, sqrt: bool = False,
+                   softsign: bool = True, storage_dtype: torch.dtype = torch.float32) -> "_MaybeQuantizedTensor":
+        """An all-zero state shaped like `ref`, without the temporary tensor and the quantise launch of
+        ``set_data(zeros_like(ref))``.  Quantising zeros gives codes 0 and scales fp16(1e-12) = 0 (ref:1006-1013,
+        2657-2676), so both forms hold the same bits."""
+        self = cls(None, try_quantize=try_quantize, signed=signed, sqrt=sqrt, softsign=softsign, storage_dtype=storage_dtype)
+        if self._try_quantize:
+            if not ref.is_cuda:
+                raise NotImplementedError(
+                    f"Attempting to quantize a non-CUDA {ref.dtype} tensor on device {ref.device} with shape "
+                    f"{tuple(ref.shape)}."
+                )
+            self._quantized = torch.zeros(ref.shape, dtype=torch.int8 if signed else torch.uint8, device=ref.device)
+            self._scales = torch.zeros((ref.numel() + 31) // 32, dtype=torch.float16, device=ref.device)
+        else:
+            self._data = torch.zeros(ref.shape, dtype=storage_dtype, device=ref.device)
+        return self
+
     def materialize(self) -> torch.Tensor:
         """The state as a float tensor: fp32 after dequantisation, or the plain tensor itself."""
         if not self.is_quantized():

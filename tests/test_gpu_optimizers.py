@@ -777,3 +777,21 @@ def test_check_numerics_with_cached_plans_and_one_scan():
     _set_grads(params, 42)
     with pytest.raises(fo.NumericsError):
         opt.step()
+
+
+@pytest.mark.parametrize("signed,sqrt,softsign", [(True, False, True), (False, True, False)])
+@pytest.mark.parametrize("quantize", [True, False])
+def test_zero_state_shortcut_equals_quantising_zeros(signed, sqrt, softsign, quantize):
+    """State creation skips the quantise launch for the all-zero start (ref:1006-1013 quantises zeros)."""
+    from flashoptim_amd.optimizers import _MaybeQuantizedTensor
+
+    for shape in [(1,), (33,), (4096, 3), (70001,)]:
+        ref = torch.empty(shape, dtype=torch.bfloat16, device=DEV)
+        kw = dict(try_quantize=quantize, signed=signed, sqrt=sqrt, softsign=softsign, storage_dtype=torch.bfloat16)
+        a = _MaybeQuantizedTensor.zeros_like(ref, **kw)
+        b = _MaybeQuantizedTensor(torch.zeros_like(ref), **kw)
+        assert a.is_quantized() == b.is_quantized() == quantize and a.shape == b.shape
+        assert parity.bits_equal(a.kernel_tensor, b.kernel_tensor) and a.kernel_tensor.dtype == b.kernel_tensor.dtype
+        if quantize:
+            assert parity.bits_equal(a.scales, b.scales) and a.scales.shape == b.scales.shape
+        assert sorted(a.state_dict("x")) == sorted(b.state_dict("x"))
