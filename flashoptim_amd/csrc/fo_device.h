@@ -81,6 +81,8 @@ __device__ __forceinline__ void load_vec(Pack<EB, EPL>& d, const void* base, int
 // Stores carry the non-temporal hint and system-scope write-through (`sc0 sc1 nt`): a streamed line goes straight
 // to memory instead of sitting dirty in L2 until it is evicted, which measures 1.5 points of HBM peak better than
 // `nt` alone on MI355X.  The compiler has no builtin for this policy on plain global stores, hence the asm.
+// (Raw buffer stores take the policy through their builtin, but buffer accesses measured 1 point slower for the
+// stores and another point for the loads than global ones in these kernels.)
 // The hazard recogniser does not look inside asm: a store of more than 64 bits must be followed by two wait
 // states before a VALU instruction may overwrite its data registers, hence the `s_nop 1` after the 128-bit form.
 #ifndef FO_STORE_WRITE_THROUGH
