@@ -270,3 +270,48 @@ def test_zero_gradients_change_nothing():
                            1e-8, 0.0, True, step)
     assert torch.equal(c.gp, p0) and m.eq(0).all() and v.eq(0).all() and c.gecc.eq(0).all()
     assert ms.eq(0).all() and vs.eq(0).all()
+
+
+def test_step_launches_can_be_captured_in_a_graph_and_replayed():
+    """The entry points only enqueue kernels on the given stream (no allocation, no memset, no synchronisation),
+    so a launch recorded into a HIP graph replays as another step.  Three replays, with eager work and
+    synchronisations in between, equal three eager launches bit for bit (Lion: the step needs no step counter)."""
+    k = _k()
+    from flashoptim_amd.launcher import BucketPlan, StepTensors
+
+    kw = MOM_MODES["lion"]
+    lens = [5000, 33, 70001]
+
+    def make(seed):
+        ps = [(_rand(n, 0.02, seed + i)).to(torch.bfloat16).to(DEV) for i, n in enumerate(lens)]
+        gs = [(_rand(n, 1e-3, seed + 10 + i)).to(torch.bfloat16).to(DEV) for i, n in enumerate(lens)]
+        es = [torch.zeros(n, dtype=torch.int8, device=DEV) for n in lens]
+        ms = [torch.zeros(n, dtype=torch.int8, device=DEV) for n in lens]
+        ss = [torch.zeros((n + 31) // 32, dtype=torch.float16, device=DEV) for n in lens]
+        return ps, gs, es, ms, ss
+
+    eager, graphed = make(3), make(3)
+    plan = BucketPlan("momentum", torch.bfloat16, 1, True,
+                      [StepTensors(p, g, e, m, s) for p, g, e, m, s in zip(*graphed)])
+    scalars = dict(lr=kw["lr"], mom_coef=kw["mom_coef"], update_coef=kw["update_coef"], weight_decay=kw["weight_decay"],
+                   decoupled=False, nesterov=False, do_lion=True)
+    plan.launch(**scalars)          # uploads the tables outside the capture; one eager step on both sides
+    for p, g, e, m, s in zip(*eager):
+        k._fused_momentum_step(m, s, p, g, e, **kw)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan.launch(**scalars)                                                    # multi-tensor launch
+        k._fused_momentum_step(graphed[3][0], graphed[4][0], graphed[0][0], graphed[1][0], graphed[2][0], **kw)  # and a single one
+    torch.cuda.synchronize()
+    for replay in range(3):
+        for p, g, e, m, s in zip(*eager):
+            k._fused_momentum_step(m, s, p, g, e, **kw)
+        k._fused_momentum_step(eager[3][0], eager[4][0], eager[0][0], eager[1][0], eager[2][0], **kw)
+        scratch = torch.randn(1 << 16, device=DEV).sum()   # unrelated eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(scratch))
+        for group_e, group_g in zip(eager, graphed):
+            for a, b in zip(group_e, group_g):
+                assert parity.bits_equal(a, b), f"replay {replay}"
