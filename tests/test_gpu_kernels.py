@@ -315,3 +315,54 @@ def test_step_launches_can_be_captured_in_a_graph_and_replayed():
         for group_e, group_g in zip(eager, graphed):
             for a, b in zip(group_e, group_g):
                 assert parity.bits_equal(a, b), f"replay {replay}"
+
+
+class _Fenced:
+    """A tensor carved out of a larger buffer whose bytes before and after it hold a canary pattern."""
+
+    PAD = 512  # bytes on each side (keeps the 16-byte alignment of the payload)
+
+    def __init__(self, n, dtype):
+        self.item = torch.empty(0, dtype=dtype).element_size()
+        self.raw = torch.full((self.PAD * 2 + n * self.item,), 0x5A, dtype=torch.uint8, device=DEV)
+        self.t = self.raw[self.PAD:self.PAD + n * self.item].view(dtype)
+        self.t.zero_()
+
+    def intact(self):
+        return bool((self.raw[:self.PAD] == 0x5A).all()) and bool((self.raw[self.raw.numel() - self.PAD:] == 0x5A).all())
+
+
+@pytest.mark.parametrize("n", [1, 31, 32, 33, 255, 256, 257, 511, 512, 513, 4095, 4096, 4097, 8191, 8193, 12288 + 40])
+def test_kernels_never_write_outside_their_tensors(n):
+    """Every state and parameter tensor sits between canary bytes; single-tensor and multi-tensor launches of every
+    kernel family (bf16 with ECC, quantised; fp32 without ECC) leave the canaries untouched."""
+    k = _k()
+    from flashoptim_amd.launcher import BucketPlan, StepTensors
+
+    groups = (n + 31) // 32
+    for dtype, ecc_dtype in ((torch.bfloat16, torch.int8), (torch.bfloat16, torch.int16), (torch.float32, None)):
+        def fenced_set():
+            f = dict(p=_Fenced(n, dtype), g=_Fenced(n, dtype), m=_Fenced(n, torch.int8), ms=_Fenced(groups, torch.float16),
+                     v=_Fenced(n, torch.uint8), vs=_Fenced(groups, torch.float16))
+            f["p"].t.copy_(_rand(n, 0.02, 1).to(dtype))
+            f["g"].t.copy_(_rand(n, 1e-3, 2).to(dtype))
+            f["e"] = None if ecc_dtype is None else _Fenced(n, ecc_dtype)
+            return f
+
+        a, b = fenced_set(), fenced_set()
+        ecc = lambda f: None if f["e"] is None else f["e"].t
+        for step in (1, 2):
+            k._fused_adam_step(a["m"].t, a["ms"].t, a["v"].t, a["vs"].t, a["p"].t, a["g"].t, ecc(a), 1e-3, 0.9, 0.999, 1e-8, 1e-5, True, step)
+        k._fused_momentum_step(a["m"].t, a["ms"].t, a["p"].t, a["g"].t, ecc(a), **MOM_MODES["lion"])
+        k._sgd_plain_step(a["p"].t, a["g"].t, ecc(a), 1e-2, 1e-4, True)
+        tensors = [StepTensors(f["p"].t, f["g"].t, ecc(f), f["m"].t, f["ms"].t, f["v"].t, f["vs"].t) for f in (a, b)]
+        ecc_bytes = 0 if ecc_dtype is None else torch.empty(0, dtype=ecc_dtype).element_size()
+        BucketPlan("adam", dtype, ecc_bytes, True, tensors).launch(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-5, decoupled=True, step=3)
+        BucketPlan("momentum", dtype, ecc_bytes, True, tensors).launch(lr=1e-2, mom_coef=0.9, update_coef=1.0, weight_decay=1e-4,
+                                                                          decoupled=False, nesterov=True, do_lion=False)
+        BucketPlan("plain", dtype, ecc_bytes, False, tensors).launch(lr=1e-2, weight_decay=1e-4, decoupled=False)
+        torch.cuda.synchronize()
+        for f in (a, b):
+            for name, fenced in f.items():
+                assert fenced is None or fenced.intact(), f"n={n} {dtype}: bytes next to `{name}` were overwritten"
+            assert bool(torch.isfinite(f["p"].t.float()).all())
