@@ -119,8 +119,11 @@ def check_master(param_gpu, ecc_gpu, param_ref, ecc_ref, what: str, step_size=No
     if pr.numel() == 0:
         return 0.0
     slack = 0.0 if step_size is None else step_size.reshape(-1).double() * STEP_REL_TOL
-    nd = (pg.double() - pr.double()).abs()
-    assert bool((nd <= ulp_of(pr) * 1.0000001 + slack).all()), f"{what}: narrow parameter off by more than one ulp"
+    # identical values agree, also where they are the same infinity or both NaN (an update that overflows the
+    # narrow dtype overflows it on both sides; inf - inf would otherwise read as a mismatch)
+    agree = (pg == pr) | (torch.isnan(pg) & torch.isnan(pr))
+    nd = torch.where(agree, torch.zeros((), dtype=torch.float64), (pg.double() - pr.double()).abs())
+    assert bool((agree | (nd <= ulp_of(pr) * 1.0000001 + slack)).all()), f"{what}: narrow parameter off by more than one ulp"
     m_ref = master_value(pr, er)
     ulp32 = ulp_of(m_ref.float())
     if er is None:
@@ -131,8 +134,11 @@ def check_master(param_gpu, ecc_gpu, param_ref, ecc_ref, what: str, step_size=No
         # is split, so two implementations can enter the split one fp32 ulp apart
         unit = ulp_of(pr) * 0.5 / (127.0 if er.dtype == torch.int8 else 32767.0)
         allowed = unit + ulp32 + slack
-    md = (master_value(pg, eg) - m_ref).abs()
-    worst = float((md / allowed).max())
+    m_gpu = master_value(pg, eg)
+    agree = (m_gpu == m_ref) | (torch.isnan(m_gpu) & torch.isnan(m_ref))
+    md = torch.where(agree, torch.zeros((), dtype=torch.float64), (m_gpu - m_ref).abs())
+    allowed = torch.where(agree, torch.ones((), dtype=torch.float64), allowed + torch.zeros_like(md))
+    worst = float(torch.where(agree, torch.zeros((), dtype=torch.float64), md / allowed).max())
     assert worst <= 1.0000001, f"{what}: master weight off by {worst:.3f} x the allowance ({float((md / unit).max()):.2f} units)"
     return worst
 
