@@ -61,15 +61,20 @@ def chunk_table(numels: Sequence[int], tiles_per_chunk: int = 0) -> tuple[torch.
 def absmax_many(tensors: Sequence[torch.Tensor]) -> list[float]:
     """``float(t.abs().max())`` of every tensor (0 for empty ones): one launch per (device, dtype) and one
     device-to-host copy per device, where the reference synchronises once per tensor
-    (``/root/reference/flashoptim/optimizers.py:656-673``).  A tensor holding a NaN reports NaN."""
+    (``/root/reference/flashoptim/optimizers.py:656-673``).  A tensor holding a NaN reports NaN.  Like the step
+    kernels it takes fp32, bf16 and fp16 tensors on a GPU; a non-contiguous tensor is compacted on the device first."""
     out: list[float] = [0.0] * len(tensors)
     groups: dict = {}
+    tensors = list(tensors)
     for i, t in enumerate(tensors):
         if t.numel() == 0:
             continue
-        if not t.is_cuda or t.dtype not in DTYPE_CODE or not t.is_contiguous():
-            out[i] = float(t.abs().max().item())  # dtypes and layouts the step kernels do not take either
-            continue
+        if not t.is_cuda:
+            raise NotImplementedError(f"absmax_many runs on a ROCm GPU only; got a tensor on {t.device}.")
+        if t.dtype not in DTYPE_CODE:
+            raise ValueError(f"Unsupported dtype {t.dtype}.")
+        if not t.is_contiguous():
+            tensors[i] = t = t.contiguous()
         groups.setdefault((t.device, t.dtype), []).append(i)
     pending = []
     for (device, dtype), idx in groups.items():

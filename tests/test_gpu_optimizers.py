@@ -732,7 +732,6 @@ def test_absmax_many_matches_torch():
     tensors.append(torch.zeros(0, dtype=torch.bfloat16, device=DEV))
     tensors.append(torch.zeros(100, dtype=torch.float32, device=DEV))
     tensors.append(torch.randn(64, 64, generator=g).to(DEV).t())                       # non-contiguous
-    tensors.append(torch.randn(5000, generator=g, dtype=torch.float64).to(DEV))         # dtype without a kernel
     big = torch.randn(3_000_000, generator=g).to(torch.bfloat16).to(DEV)
     tensors.append(big[3:])                                                             # 2-byte aligned view
     spike = torch.zeros(70000, dtype=torch.float16, device=DEV); spike[-1] = -60000.0
@@ -746,6 +745,10 @@ def test_absmax_many_matches_torch():
     nan = torch.ones(5000, dtype=torch.bfloat16, device=DEV); nan[4000] = float("nan")
     import math
     assert math.isnan(kernels.absmax_many([nan])[0])
+    with pytest.raises(ValueError):
+        kernels.absmax_many([torch.zeros(8, dtype=torch.float64, device=DEV)])
+    with pytest.raises(NotImplementedError):
+        kernels.absmax_many([torch.zeros(8)])
 
 
 def test_check_numerics_with_cached_plans_and_one_scan():
