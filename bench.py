@@ -95,6 +95,30 @@ def make_params(shapes, dtype, device, grad_scales=None, seed=0):
     return params
 
 
+def rotating_gradients(params, step, device, grad_scales=None, sets=3):
+    """Gradients are redrawn for every step, as in training: `sets` gradient lists are drawn once (seeds 1000 + k,
+    outside the timed region) and the returned step function installs the next list as ``p.grad`` before each
+    ``step()``, so gradient values and addresses change from step to step."""
+    rings = []
+    for k in range(sets):
+        torch.manual_seed(1000 + k)
+        ring = []
+        for i, p in enumerate(params):
+            s = 1.0 if grad_scales is None else grad_scales[i]
+            ring.append((torch.randn(p.shape, device=device, dtype=torch.float32) * (1e-3 * s)).to(p.dtype))
+        rings.append(ring)
+    counter = [0]
+
+    def run():
+        ring = rings[counter[0] % sets]
+        counter[0] += 1
+        for p, g in zip(params, ring):
+            p.grad = g
+        step()
+
+    return run
+
+
 def build_workload(name: str, device):
     import flashoptim_amd as fo
 
@@ -106,8 +130,10 @@ def build_workload(name: str, device):
         params = make_params(shapes, torch.bfloat16, device, scales)
         mwb = 24 if name.endswith("24") else 32
         opt = fo.FlashAdamW(params, master_weight_bits=mwb, **hp)
-        return dict(params=params, opt=opt, step=opt.step, bpp=bytes_per_param(2, 1 if mwb == 24 else 2, 2),
-                    desc=f"Llama-3-8B-shaped parameter list, bf16, FlashAdamW, master_weight_bits={mwb}",
+        return dict(params=params, opt=opt, step=rotating_gradients(params, opt.step, device, scales),
+                    bpp=bytes_per_param(2, 1 if mwb == 24 else 2, 2),
+                    desc=f"Llama-3-8B-shaped parameter list, bf16, FlashAdamW, master_weight_bits={mwb}, "
+                         "gradients redrawn per step (3 rotating sets)",
                     launch="one multi-tensor launch per step", optimizer="FlashAdamW", mwb=mwb)
     if name in ("llama8b-lion", "llama8b-sgdw"):
         shapes = llama3_8b_shapes()
@@ -124,8 +150,9 @@ def build_workload(name: str, device):
     if name == "flat-2p30":
         params = make_params([("flat", (1 << 30,))], torch.bfloat16, device)
         opt = fo.FlashAdamW(params, master_weight_bits=24, **hp)
-        return dict(params=params, opt=opt, step=opt.step, bpp=bytes_per_param(2, 1, 2),
-                    desc="one flat bf16 tensor of 2^30 elements, FlashAdamW, master_weight_bits=24",
+        return dict(params=params, opt=opt, step=rotating_gradients(params, opt.step, device), bpp=bytes_per_param(2, 1, 2),
+                    desc="one flat bf16 tensor of 2^30 elements, FlashAdamW, master_weight_bits=24, gradients redrawn per "
+                         "step (3 rotating sets)",
                     launch="one single-tensor launch per step", optimizer="FlashAdamW", mwb=24)
     if name in ("ragged-lion", "ragged-sgdw"):
         lens = ragged_lengths()
