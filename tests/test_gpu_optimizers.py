@@ -798,3 +798,40 @@ def test_zero_state_shortcut_equals_quantising_zeros(signed, sqrt, softsign, qua
         if quantize:
             assert parity.bits_equal(a.scales, b.scales) and a.scales.shape == b.scales.shape
         assert sorted(a.state_dict("x")) == sorted(b.state_dict("x"))
+
+
+def test_pooled_step_counters_behave_like_separate_scalars():
+    """Adam's per-parameter CPU `step` scalars are views into one pooled tensor while a cached plan is live; they
+    still read, checkpoint and advance like the separate fp32 scalars of the reference (ref:1846-1853)."""
+    fo = _fo()
+    params = _make_params([4096, 1000, 33, 70001], torch.bfloat16, 6)
+    opt = fo.FlashAdamW(params, lr=1e-3)
+    for it in range(4):
+        _set_grads(params, 60 + it)
+        opt.step()
+    assert [float(opt.state[p]["step"]) for p in params] == [4.0] * 4
+    sd = opt.state_dict()
+    for idx in sd["state"]:
+        step = sd["state"][idx]["step"]
+        assert step.dtype == torch.float32 and step.device.type == "cpu" and step.dim() == 0
+        assert step.untyped_storage().nbytes() == 4, "checkpointed counters must not drag the pool along"
+    # one parameter stepped on its own moves only its counter, and the next full step keeps them apart
+    _set_grads(params, 70)
+    opt.step_param(params[1])
+    assert [float(opt.state[p]["step"]) for p in params] == [4.0, 5.0, 4.0, 4.0]
+    params[1].grad = None
+    opt.step()
+    opt.step()   # second call runs from the rebuilt cache
+    assert [float(opt.state[p]["step"]) for p in params] == [6.0, 5.0, 6.0, 6.0]
+    # a reloaded optimizer continues from the saved counters
+    fresh_params = [nn.Parameter(p.detach().clone()) for p in params]
+    fresh = fo.FlashAdamW(fresh_params, lr=1e-3)
+    fresh.load_state_dict(copy.deepcopy(opt.state_dict()))
+    for a, b in zip(params, fresh_params):
+        a.grad = torch.ones_like(a) * 1e-3
+        b.grad = a.grad.clone()
+    opt.step()
+    fresh.step()
+    assert [float(fresh.state[p]["step"]) for p in fresh_params] == [7.0, 6.0, 7.0, 7.0]
+    for a, b in zip(params, fresh_params):  # the uncompressed bf16 checkpoint requantises the moments: close, not equal
+        torch.testing.assert_close(a.float(), b.float(), rtol=0, atol=2e-3)
