@@ -594,7 +594,27 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         restored["error_bits"] = errs
         return restored
 
+    def __getstate__(self) -> dict[str, Any]:
+        """For ``copy.deepcopy`` / ``pickle`` of the optimizer object itself: torch keeps ``defaults``, ``state`` and
+        ``param_groups``; the scalar configuration of this class and its subclasses travels along."""
+        state = super().__getstate__()
+        state["_flash_config"] = {k: v for k, v in self.__dict__.items()
+                                  if k.startswith("_") and isinstance(v, (bool, int, float, str, type(None)))}
+        return state
+
     def __setstate__(self, state: dict[str, Any]) -> None:
+        if "_flash_config" in state:
+            # a copied / unpickled optimizer: its states are live containers already, nothing to convert; hooks of
+            # the original are not copied, launch caches and statistics are keyed by object identity
+            state = dict(state)
+            config = state.pop("_flash_config")
+            super().__setstate__(state)
+            self.__dict__.update(config)
+            self._gradient_release = False
+            self._plan_epoch = int(config.get("_plan_epoch", 0)) + 1
+            self._group_cache = {}
+            self._transient_state = {}
+            return
         opt_state = cast(dict[torch.Tensor, Any], state["state"])
         for group in cast(list[dict[str, Any]], state["param_groups"]):
             for param in group["params"]:

@@ -835,3 +835,26 @@ def test_pooled_step_counters_behave_like_separate_scalars():
     assert [float(fresh.state[p]["step"]) for p in fresh_params] == [7.0, 6.0, 7.0, 7.0]
     for a, b in zip(params, fresh_params):  # the uncompressed bf16 checkpoint requantises the moments: close, not equal
         torch.testing.assert_close(a.float(), b.float(), rtol=0, atol=2e-3)
+
+
+def test_deepcopy_of_the_optimizer_is_an_independent_working_optimizer():
+    fo = _fo()
+    params = _make_params([4096, 33, 70001], torch.bfloat16, 9)
+    opt = fo.FlashAdamW(params, lr=1e-3, weight_decay=0.01)
+    for it in range(2):
+        _set_grads(params, 80 + it)
+        opt.step()
+    twin = copy.deepcopy(opt)           # copies parameters, gradients and states
+    twin_params = twin.param_groups[0]["params"]
+    assert all(a is not b and torch.equal(a, b) for a, b in zip(params, twin_params))
+    assert twin._quantize == opt._quantize and twin._master_bytewidth == opt._master_bytewidth and not twin._gradient_release
+    for it in range(2):
+        _set_grads(params, 90 + it)
+        for a, b in zip(params, twin_params):
+            b.grad = a.grad.clone()
+        opt.step()
+        twin.step()
+    for a, b in zip(params, twin_params):
+        assert torch.equal(a, b)
+        assert torch.equal(opt.state[a]["exp_avg"].quantized, twin.state[b]["exp_avg"].quantized)
+        assert float(twin.state[b]["step"]) == 4.0
