@@ -7,6 +7,7 @@ raw ``data_ptr()`` values and the current HIP stream, and return immediately aft
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import os
 import threading
@@ -108,7 +109,20 @@ def check(rc: int, what: str) -> None:
 
 
 def current_stream_ptr(device: torch.device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """Raw handle of torch's current stream on `device` (what the launches are enqueued on)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    return torch._C._cuda_getCurrentRawStream(index)
+
+
+_NO_GUARD = contextlib.nullcontext()
+
+
+def device_guard(device: torch.device):
+    """Context that makes `device` current for the HIP calls inside it; free when it already is (the usual case:
+    ``torch.cuda.device`` costs several microseconds per launch)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(device)
 
 
 def ptr(t: Optional[torch.Tensor]) -> Optional[int]:

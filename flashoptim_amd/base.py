@@ -151,6 +151,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         self._transient_state: dict[int, dict[str, Any]] = {}  # id(param) -> {"maxabs": ...}; never serialised
         self._gradient_release = False
         self._plan_epoch = 0                       # bumped whenever cached launch plans may be stale
+        self._state_ready: set[int] = set()        # id(param) of parameters whose state tensors exist
         self._group_cache: dict[int, _GroupCache] = {}
 
         group_defaults = dict(defaults or {})
@@ -325,7 +326,9 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
 
     def _plan_param(self, p: torch.Tensor, group: dict[str, Any]) -> Optional[tuple[LaunchKey, StepTensors]]:
         """Everything ``step_param`` does short of launching (ref:699-759)."""
-        self._ensure_state_initialized(p, hparams=group)
+        if id(p) not in self._state_ready or not self.state.get(p):
+            self._ensure_state_initialized(p, hparams=group)
+            self._state_ready.add(id(p))
         param_state = self.state[p]
         if p.numel() < 1:
             return None  # state exists (checkpoint logic wants it) but there is nothing to update
@@ -614,6 +617,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
             self._plan_epoch = int(config.get("_plan_epoch", 0)) + 1
             self._group_cache = {}
             self._transient_state = {}
+            self._state_ready = set()
             return
         opt_state = cast(dict[torch.Tensor, Any], state["state"])
         for group in cast(list[dict[str, Any]], state["param_groups"]):
@@ -629,6 +633,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         # state tensors were replaced: cached pointer tables and step counters are stale
         self._plan_epoch = getattr(self, "_plan_epoch", 0) + 1
         self._group_cache = {}
+        self._state_ready = set()
 
     def load_state_dict(self, state_dict: dict[str, Any]) -> None:
         """Also accepts checkpoints of the stock torch optimizers, which may lack ``initial_lr`` (ref:974-986)."""

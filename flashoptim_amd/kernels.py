@@ -77,7 +77,7 @@ def quantize(
     if out_scales.numel() < (n + GROUP_SIZE - 1) // GROUP_SIZE or out_scales.dtype != torch.float16:
         raise ValueError("out_scales must be fp16 with at least ceil(N/32) elements")
     if n > 0:
-        with torch.cuda.device(x.device):
+        with _native.device_guard(x.device):
             rc = _native.lib().fo_quantize(
                 x.data_ptr(), DTYPE_CODE[x.dtype], out_int8.data_ptr(), out_scales.data_ptr(), n,
                 int(signed), int(sqrt), int(softsign), _native.current_stream_ptr(x.device),
@@ -112,7 +112,7 @@ def dequantize(
     if out_float.dtype != torch.float32 or out_float.numel() != n or not out_float.is_contiguous():
         raise ValueError("out_float must be a contiguous fp32 tensor with as many elements as the codes")
     if n > 0:
-        with torch.cuda.device(codes.device):
+        with _native.device_guard(codes.device):
             rc = _native.lib().fo_dequantize(
                 codes.data_ptr(), scales.data_ptr(), out_float.data_ptr(), n, int(signed), int(sqrt),
                 int(softsign), _native.current_stream_ptr(codes.device),
@@ -143,7 +143,7 @@ def reconstruct_fp32_param(param: torch.Tensor, error_bits: torch.Tensor) -> tor
     if n > 0:
         narrow = param.contiguous()
         ecc = error_bits.contiguous()
-        with torch.cuda.device(param.device):
+        with _native.device_guard(param.device):
             rc = _native.lib().fo_ecc_join(
                 narrow.data_ptr(), DTYPE_CODE[param.dtype], ecc.data_ptr(), ecc.element_size(), out.data_ptr(), n,
                 _native.current_stream_ptr(param.device),
@@ -178,7 +178,7 @@ def compute_ecc_bits(
     if n > 0:
         x = fp32_param.to(narrow_param.device).contiguous()
         narrow = narrow_param.contiguous()
-        with torch.cuda.device(narrow.device):
+        with _native.device_guard(narrow.device):
             rc = _native.lib().fo_ecc_split(
                 x.data_ptr(), narrow.data_ptr(), DTYPE_CODE[narrow.dtype], out.data_ptr(), num_err_bytes, n,
                 _native.current_stream_ptr(narrow.device),
@@ -230,7 +230,7 @@ def _fused_adam_step(
         return
     _check_step_tensors(param, grad, errors)
     ecc_bytes = _ecc_bytes(errors)
-    with torch.cuda.device(param.device):
+    with _native.device_guard(param.device):
         rc = _native.lib().fo_adam_step(
             mom.data_ptr(), mom_scales_f16.data_ptr() if quantize_optim_states else None,
             var.data_ptr(), var_scales_f16.data_ptr() if quantize_optim_states else None,
@@ -264,7 +264,7 @@ def _fused_momentum_step(
         return
     _check_step_tensors(param, grad, errors)
     ecc_bytes = _ecc_bytes(errors)
-    with torch.cuda.device(param.device):
+    with _native.device_guard(param.device):
         rc = _native.lib().fo_momentum_step(
             momentum.data_ptr(), scales_f16.data_ptr() if quantize_optim_states else None, param.data_ptr(),
             grad.data_ptr(), _native.ptr(errors), n, DTYPE_CODE[param.dtype], ecc_bytes,
@@ -288,7 +288,7 @@ def _sgd_plain_step(
     if n == 0:
         return
     _check_step_tensors(param, grad, errors)
-    with torch.cuda.device(param.device):
+    with _native.device_guard(param.device):
         rc = _native.lib().fo_sgd_plain_step(
             param.data_ptr(), grad.data_ptr(), _native.ptr(errors), n, DTYPE_CODE[param.dtype], _ecc_bytes(errors),
             lr, weight_decay, int(decoupled), _native.current_stream_ptr(param.device),
@@ -309,6 +309,6 @@ def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
     nbytes = src.numel() * src.element_size()
     if dst.numel() * dst.element_size() != nbytes:
         raise ValueError("dst and src must have the same size in bytes")
-    with torch.cuda.device(src.device):
+    with _native.device_guard(src.device):
         rc = _native.lib().fo_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes, _native.current_stream_ptr(src.device))
     _native.check(rc, "fo_copy_bytes")

@@ -82,7 +82,7 @@ def absmax_many(tensors: Sequence[torch.Tensor]) -> list[float]:
         for d, i in zip(table, idx):
             d.param, d.n = tensors[i].data_ptr(), tensors[i].numel()
         chunks_host, n_chunks = chunk_table([tensors[i].numel() for i in idx], tiles_per_chunk=16)
-        with torch.cuda.device(device):
+        with _native.device_guard(device):
             descs = torch.frombuffer(bytearray(bytes(table)), dtype=torch.uint8).to(device)
             chunks = chunks_host.to(device)
             result = torch.zeros(len(idx), dtype=torch.float32, device=device)
@@ -139,7 +139,7 @@ class BucketPlan:
         """Enqueue the bucket's kernel on the current stream with the given fp32 scalars."""
         if self.n_chunks == 0:
             return
-        with torch.cuda.device(self.device):
+        with _native.device_guard(self.device):
             if self._dirty:
                 self._upload()
             lib = _native.lib()
