@@ -219,7 +219,7 @@ static void state_store_group(void *state, uint16_t *scales, int quantized, int 
         for (int k = 0; k < cnt; ++k) store_narrow(state, dtype, base + k, vals[k]);
         return;
     }
-    float tmp[FO_GROUP]; int32_t q[FO_GROUP];
+    float tmp[FO_GROUP] = {0.0f}; int32_t q[FO_GROUP];
     for (int k = 0; k < cnt; ++k) tmp[k] = do_sqrt ? sqrtf(vals[k]) : vals[k];   /* ref:2393 */
     float amax = quant_group(tmp, cnt, is_signed, softsign, q);
     for (int k = 0; k < cnt; ++k) {
