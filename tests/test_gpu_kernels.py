@@ -418,3 +418,36 @@ def test_randomised_configurations_match_oracle():
                 info = T.momentum_step_ref(c.states[0], c.p, g, c.ecc, **kw)
             c.compare(f"{what} step={step}", info)
             c.resync_oracle()
+
+
+def test_the_binding_shown_in_the_integration_notes_runs():
+    """The ctypes stub printed in INTEGRATION.md (what a maintainer of the reference would add) is executed as
+    written, against the built library, and gives the same bits as this package's own binding."""
+    import os
+    import re
+
+    from flashoptim_amd import _native
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "INTEGRATION.md")).read()
+    block = re.search(r"```python\n(.*?)```", text, re.S).group(1)
+    block = "\n".join(line[3:] if line.startswith("   ") else line for line in block.splitlines())
+    block = block.replace('ctypes.CDLL("libflashoptim_hip.so")', f'ctypes.CDLL({_native.library_path()!r})')
+    scope = {}
+    exec(compile(block, "INTEGRATION.md", "exec"), scope)
+    k = _k()
+    n = 10000 + 17
+
+    def tensors():
+        p = _rand(n, 0.02, 1).to(torch.bfloat16).to(DEV)
+        g = _rand(n, 1e-3, 2).to(torch.bfloat16).to(DEV)
+        return (torch.zeros(n, dtype=torch.int8, device=DEV), torch.zeros((n + 31) // 32, dtype=torch.float16, device=DEV),
+                torch.zeros(n, dtype=torch.uint8, device=DEV), torch.zeros((n + 31) // 32, dtype=torch.float16, device=DEV),
+                p, g, torch.zeros(n, dtype=torch.int8, device=DEV))
+
+    a, b = tensors(), tensors()
+    for step in (1, 2):
+        scope["_fused_adam_step"](*a, 1e-3, 0.9, 0.999, 1e-8, 1e-5, True, step)
+        k._fused_adam_step(*b, 1e-3, 0.9, 0.999, 1e-8, 1e-5, True, step)
+    for x, y in zip(a, b):
+        assert parity.bits_equal(x, y)
