@@ -17,7 +17,20 @@ __device__ __forceinline__ u32 absmax_of_range(const void* x, int64_t begin, int
     constexpr int EPL = DTypeInfo<DT>::epl;
     constexpr int EB = DTypeInfo<DT>::bytes;
     u32 best = 0;
-    for (int64_t first = begin + (int64_t)threadIdx.x * EPL; first < end; first += (int64_t)kStatsThreads * EPL) {
+    constexpr int64_t kStride = (int64_t)kStatsThreads * EPL;
+    int64_t first = begin + (int64_t)threadIdx.x * EPL;
+    if (aligned) {  // four independent loads in flight per thread while whole strides remain
+        for (; first + 3 * kStride + EPL <= end; first += 4 * kStride) {
+            Pack<EB, EPL> raw[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) load_vec<EB, EPL>(raw[j], x, first + j * kStride);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int k = 0; k < EPL; ++k) best = max(best, as_u32(widen<DT, EPL>(raw[j], k)) & 0x7fffffffu);
+        }
+    }
+    for (; first < end; first += kStride) {
         Pack<EB, EPL> raw;
         if (aligned && first + EPL <= end) load_vec<EB, EPL>(raw, x, first);
         else load_guarded<EB, EPL>(raw, x, first, end);
