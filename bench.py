@@ -274,6 +274,10 @@ def main() -> None:
         raise SystemExit("bench.py needs a ROCm GPU")
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if not os.path.exists(os.path.join(ROOT, "flashoptim_amd", "lib", "libflashoptim_hip.so")):
+        import __graft_entry__
+
+        __graft_entry__.build()  # loads what is built; builds only when nothing is
 
     work = build_workload(args.workload, device)
     step = work["step"]

@@ -10,6 +10,13 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # the tests load what is built; only when nothing is built yet do they build (hipcc cross-compiles without a GPU)
+    lib = os.path.join(ROOT, "flashoptim_amd", "lib", "libflashoptim_hip.so")
+    if not os.path.exists(lib):
+        import subprocess
+
+        subprocess.run(["make", "-j", "8", "-C", os.path.join(ROOT, "flashoptim_amd", "csrc")], check=True,
+                       capture_output=True)
 
 
 def pytest_collection_modifyitems(config, items):
