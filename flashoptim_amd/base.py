@@ -80,6 +80,7 @@ class _GroupCache:
     params: list
     signature: Any
     buckets: list
+    idle: list                        # non-empty parameters that had no gradient (or are frozen) when the cache was built
     # check_numerics: log2 of the coarsest weight resolution over the group's parameters (None: nothing to check)
     numerics_needed: Optional[float] = None
 
@@ -385,9 +386,10 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
     # -- step(): one multi-tensor launch per bucket, with the host work of an unchanged group cached ------------
     def _step_group_slow(self, index: int, group: dict[str, Any]) -> None:
         """Full per-parameter planning (state creation, checks, counters), then one launch per bucket; leaves a
-        cache behind when every parameter of the group took part."""
+        cache behind that stays valid while the same parameters have gradients (frozen or unused ones sit out)."""
         planned: dict[LaunchKey, list] = {}
-        complete = True
+        cacheable = True
+        idle = []
         if self._check_numerics:  # one scan for every parameter that has no cached statistic yet
             missing = [p for p in group["params"]
                        if p.grad is not None and self._transient_state.get(id(p), {}).get("maxabs") is None]
@@ -396,12 +398,13 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         for p in group["params"]:
             plan = self._plan_param(p, group)
             if plan is None:
-                complete = False
+                if p.numel() > 0:
+                    idle.append(p)
                 continue
             key, tensors = plan
             planned.setdefault(key, []).append((p, tensors))
             if tensors.param is not p:
-                complete = False  # sharded wrapper: keep the generic path
+                cacheable = False  # sharded wrapper: keep the generic path
         buckets = []
         for key, items in planned.items():
             tensors = [t for _, t in items]
@@ -424,19 +427,23 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
                 t.grad = None  # the cache must not keep gradients alive
             buckets.append(_Bucket(key.kind, key.dtype, key.ecc_bytes, key.quantized, [p for p, _ in items], tensors,
                                    plan, step_pool, scalars.get("step")))
-        if complete and buckets:
+        if cacheable and buckets:
             needed = None
             if self._check_numerics:
-                each = [self._numerics_needed(p, group["master_bytewidth"]) for p in group["params"]]
+                each = [self._numerics_needed(p, group["master_bytewidth"]) for b in buckets for p in b.params]
                 needed = max((x for x in each if x is not None), default=None)
             self._group_cache[index] = _GroupCache(self._plan_epoch, list(group["params"]),
-                                                   self._plan_signature(group), buckets, needed)
+                                                   self._plan_signature(group), buckets, idle, needed)
         else:
             self._group_cache.pop(index, None)
 
     def _step_group_fast(self, cache: _GroupCache, group: dict[str, Any]) -> bool:
-        """Re-issue the cached launches of a group whose parameters all have gradients of the cached layout.
-        Returns False (having changed nothing) when the group must go through the full path instead."""
+        """Re-issue the cached launches of a group whose parameters have gradients of the cached layout (and whose
+        idle parameters still have none).  Returns False (having changed nothing) when the group must go through
+        the full path instead."""
+        for p in cache.idle:
+            if p.grad is not None and p.requires_grad:
+                return False
         moved = []
         for b in cache.buckets:
             ptrs = b.plan.grad_ptrs if b.plan is not None else None
@@ -445,6 +452,8 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
                 if g is None or not p.requires_grad:
                     return False
                 if ptrs is not None:
+                    if p.data_ptr() != b.plan.param_ptrs[i]:
+                        return False  # the parameter's storage was replaced (p.data = ..., module.to(...))
                     ptr = g.data_ptr()
                     if ptr != ptrs[i]:
                         if g.dtype != b.dtype or g.device != p.device or not g.is_contiguous() or g.numel() != p.numel():

@@ -117,6 +117,7 @@ class BucketPlan:
         # the state tensors must outlive the table that points at them (gradients are tracked by address only)
         self._keepalive = [(t.param, t.ecc, t.mom, t.mom_scales, t.var, t.var_scales) for t in tensors]
         self.grad_ptrs = [d.grad for d in self.table]
+        self.param_ptrs = [d.param for d in self.table]
 
         host, self.n_chunks = chunk_table(numels, tiles_per_chunk)
         self.chunks_dev = host.to(self.device)

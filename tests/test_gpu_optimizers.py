@@ -322,7 +322,7 @@ def test_check_numerics_raises_when_lr_cannot_move_the_weights():
                     warnings.simplefilter("ignore")
                     opt = fo.FlashLion([w], lr=lr, check_numerics=True, master_weight_bits=mwb)
                 w.grad = torch.ones_like(w)
-                need = _log2_min_expressible_step_size(torch.bfloat16, float(w.abs().max()), _BITS_TO_BYTES[mwb])
+                need = _log2_min_expressible_step_size(torch.bfloat16, float(w.detach().abs().max()), _BITS_TO_BYTES[mwb])
                 if math.log2(lr) < need:
                     with pytest.raises(fo.NumericsError):
                         opt.step()
@@ -695,6 +695,76 @@ def test_cached_step_plan_follows_moving_missing_and_freed_gradients():
     del hold
     gc.collect()
     assert ref() is None, "the optimizer's cached plan kept a gradient alive"
+
+
+def _count_full_plans(opt):
+    """Wrap the optimizer's full planning path with a call counter."""
+    calls = []
+    full = opt._step_group_slow
+
+    def counted(index, group):
+        calls.append(index)
+        return full(index, group)
+
+    opt._step_group_slow = counted
+    return calls
+
+
+def test_cached_step_plan_with_frozen_and_unused_parameters():
+    """A group that holds a frozen parameter and one that never receives a gradient (fine-tuning) still steps from
+    the cached plan; the cache is dropped the moment the unused parameter gets a gradient, and the result stays
+    bit-identical to per-tensor stepping."""
+    fo = _fo()
+    shapes = [5000, 33, 4096, 70001, 0]
+    pa, pb = _make_params(shapes, torch.bfloat16, 33), _make_params(shapes, torch.bfloat16, 33)
+    for params in (pa, pb):
+        params[1].requires_grad_(False)
+    oa, ob = fo.FlashAdamW(pa, lr=1e-3), fo.FlashAdamW(pb, lr=1e-3)
+    full_plans = _count_full_plans(oa)
+    frozen_before = pa[1].clone()
+    for it in range(6):
+        for params in (pa, pb):
+            _set_grads(params, 300 + it)
+            params[1].grad = None
+            if it < 4:
+                params[2].grad = None           # unused until the fifth step
+        oa.step()
+        for p in pb:
+            ob.step_param(p)
+        if it == 3:
+            assert full_plans == [0], "steps 2-4 should have come from the cached plan"
+    assert full_plans == [0, 0], "one full plan at the start and one when the unused parameter joined"
+    assert torch.equal(pa[1], frozen_before)
+    for a, b in zip(pa, pb):
+        assert torch.equal(a, b)
+        sa, sb = _state_tensors(oa, a), _state_tensors(ob, b)
+        for k in sa:
+            assert parity.bits_equal(sa[k], sb[k]), k
+    assert oa.state[pa[0]]["step"].item() == 6 and oa.state[pa[2]]["step"].item() == 2
+
+
+def test_cached_step_plan_notices_replaced_parameter_storage():
+    """`p.data = ...` (what module.to() and friends do) moves a parameter to new memory; the cached launch table
+    must not go on updating the old block."""
+    fo = _fo()
+    shapes = [5000, 4096, 70001]
+    pa, pb = _make_params(shapes, torch.bfloat16, 34), _make_params(shapes, torch.bfloat16, 34)
+    oa, ob = fo.FlashAdamW(pa, lr=1e-3), fo.FlashAdamW(pb, lr=1e-3)
+    old_block = None
+    for it in range(4):
+        _set_grads(pa, 400 + it)
+        _set_grads(pb, 400 + it)
+        if it == 2:
+            old_block = pa[1].data
+            pa[1].data = old_block.clone()
+            assert pa[1].data_ptr() != old_block.data_ptr()
+            old_copy = old_block.clone()
+        oa.step()
+        for p in pb:
+            ob.step_param(p)
+    assert torch.equal(old_block, old_copy), "the step wrote into the parameter's previous storage"
+    for a, b in zip(pa, pb):
+        assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("dtype,mwb", [(torch.bfloat16, 24), (torch.bfloat16, 32), (torch.float32, None), (torch.float16, None)])
