@@ -29,6 +29,12 @@ def _require_device(t: torch.Tensor, what: str) -> None:
         )
 
 
+def _require_same_device(ref: torch.Tensor, other: Optional[torch.Tensor], what: str) -> None:
+    """The kernels dereference raw addresses: a tensor on another device (or the host) would fault the GPU."""
+    if other is not None and other.device != ref.device:
+        raise ValueError(f"{what} is on {other.device}, expected {ref.device}.")
+
+
 def _ecc_bytes(errors: Optional[torch.Tensor]) -> int:
     """Width of the correction term: 0 (none), 1 (int8, 24-bit master) or 2 (int16, 32-bit master);
     same rule as ``_ecc_kernel_params`` (ref:1514-1524)."""
@@ -74,8 +80,11 @@ def quantize(
         out_scales = torch.empty((n + GROUP_SIZE - 1) // GROUP_SIZE, device=x.device, dtype=torch.float16)
     if out_int8.numel() != n or not out_int8.is_contiguous() or out_int8.element_size() != 1:
         raise ValueError("out_int8 must be a contiguous 1-byte tensor with as many elements as the input")
-    if out_scales.numel() < (n + GROUP_SIZE - 1) // GROUP_SIZE or out_scales.dtype != torch.float16:
-        raise ValueError("out_scales must be fp16 with at least ceil(N/32) elements")
+    if (out_scales.numel() < (n + GROUP_SIZE - 1) // GROUP_SIZE or out_scales.dtype != torch.float16
+            or not out_scales.is_contiguous()):
+        raise ValueError("out_scales must be contiguous fp16 with at least ceil(N/32) elements")
+    _require_same_device(x, out_int8, "out_int8")
+    _require_same_device(x, out_scales, "out_scales")
     if n > 0:
         with _native.device_guard(x.device):
             rc = _native.lib().fo_quantize(
@@ -111,6 +120,8 @@ def dequantize(
         out_float = torch.empty_like(codes, dtype=torch.float32)
     if out_float.dtype != torch.float32 or out_float.numel() != n or not out_float.is_contiguous():
         raise ValueError("out_float must be a contiguous fp32 tensor with as many elements as the codes")
+    _require_same_device(codes, scales, "in_scales")
+    _require_same_device(codes, out_float, "out_float")
     if n > 0:
         with _native.device_guard(codes.device):
             rc = _native.lib().fo_dequantize(
@@ -138,6 +149,7 @@ def reconstruct_fp32_param(param: torch.Tensor, error_bits: torch.Tensor) -> tor
     _require_device(param, "reconstruct_fp32_param")
     if error_bits.numel() != param.numel():
         raise ValueError("error_bits must have as many elements as param")
+    _require_same_device(param, error_bits, "error_bits")
     out = torch.empty(param.shape, dtype=torch.float32, device=param.device)
     n = param.numel()
     if n > 0:
@@ -191,6 +203,7 @@ def compute_ecc_bits(
 
 
 def _check_step_tensors(param: torch.Tensor, grad: torch.Tensor, errors: Optional[torch.Tensor]) -> None:
+    """Everything the step kernels assume about param / grad / ECC and cannot check from raw addresses."""
     _require_device(param, "fused step")
     if param.dtype not in DTYPE_CODE:
         raise ValueError(f"Unsupported parameter dtype {param.dtype}.")
@@ -200,8 +213,35 @@ def _check_step_tensors(param: torch.Tensor, grad: torch.Tensor, errors: Optiona
         raise ValueError("grad and param must have the same number of elements")
     if grad.device != param.device:
         raise ValueError("grad and param must be on the same device")
-    if errors is not None and errors.numel() != param.numel():
-        raise ValueError("error_bits and param must have the same number of elements")
+    if not param.is_contiguous() or not grad.is_contiguous():
+        raise RuntimeError("the fused kernels need contiguous param and grad tensors")
+    if errors is not None:
+        if errors.numel() != param.numel():
+            raise ValueError("error_bits and param must have the same number of elements")
+        if not errors.is_contiguous():
+            raise RuntimeError("the fused kernels need a contiguous error_bits tensor")
+        _require_same_device(param, errors, "error_bits")
+
+
+def _check_moment(param: torch.Tensor, values: torch.Tensor, scales: Optional[torch.Tensor], quantized: bool,
+                  signed: bool, name: str) -> None:
+    """One optimizer state as the step kernels read and write it: 8-bit codes with fp16 group scales, or a tensor
+    of the parameter's dtype."""
+    n = param.numel()
+    if values.numel() != n or not values.is_contiguous():
+        raise ValueError(f"{name} must be contiguous with as many elements as param ({n}), got {values.numel()}.")
+    _require_same_device(param, values, name)
+    if not quantized:
+        if values.dtype != param.dtype:
+            raise ValueError(f"unquantised {name} must have the parameter's dtype {param.dtype}, got {values.dtype}.")
+        return
+    if values.dtype != (torch.int8 if signed else torch.uint8):
+        raise ValueError(f"quantised {name} must be {'int8' if signed else 'uint8'}, got {values.dtype}.")
+    if scales is None or scales.dtype != torch.float16 or not scales.is_contiguous():
+        raise ValueError(f"{name} scales must be a contiguous fp16 tensor.")
+    if scales.numel() < (n + GROUP_SIZE - 1) // GROUP_SIZE:
+        raise ValueError(f"{name} scales hold {scales.numel()} groups, {(n + GROUP_SIZE - 1) // GROUP_SIZE} needed.")
+    _require_same_device(param, scales, f"{name} scales")
 
 
 def _fused_adam_step(
@@ -229,6 +269,8 @@ def _fused_adam_step(
     if n == 0:
         return
     _check_step_tensors(param, grad, errors)
+    _check_moment(param, mom, mom_scales_f16, quantize_optim_states, True, "mom")
+    _check_moment(param, var, var_scales_f16, quantize_optim_states, False, "var")
     ecc_bytes = _ecc_bytes(errors)
     with _native.device_guard(param.device):
         rc = _native.lib().fo_adam_step(
@@ -263,6 +305,7 @@ def _fused_momentum_step(
     if n == 0:
         return
     _check_step_tensors(param, grad, errors)
+    _check_moment(param, momentum, scales_f16, quantize_optim_states, True, "momentum")
     ecc_bytes = _ecc_bytes(errors)
     with _native.device_guard(param.device):
         rc = _native.lib().fo_momentum_step(
@@ -306,9 +349,13 @@ def absmax_many(tensors) -> list:
 def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
     """Device copy with the step kernels' access shape; a measurement aid (counter calibration, attainable
     streaming rate)."""
+    _require_device(src, "copy_bytes")
+    _require_same_device(src, dst, "dst")
     nbytes = src.numel() * src.element_size()
     if dst.numel() * dst.element_size() != nbytes:
         raise ValueError("dst and src must have the same size in bytes")
+    if not src.is_contiguous() or not dst.is_contiguous():
+        raise ValueError("copy_bytes needs contiguous tensors")
     with _native.device_guard(src.device):
         rc = _native.lib().fo_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes, _native.current_stream_ptr(src.device))
     _native.check(rc, "fo_copy_bytes")

@@ -25,7 +25,7 @@ from typing import Optional, Sequence
 
 import torch
 
-from . import _native
+from . import _native, kernels
 from ._native import DTYPE_CODE, FoChunk, FoTensorDesc
 
 
@@ -108,6 +108,14 @@ class BucketPlan:
         if any(t.param.device != self.device for t in tensors):
             raise ValueError("all tensors of one multi-tensor launch must live on one device")
         self.n_tensors = len(tensors)
+        for t in tensors:  # once per plan: the kernels only see addresses and trust these shapes
+            kernels._check_step_tensors(t.param, t.grad, t.ecc)
+            if kernels._ecc_bytes(t.ecc) != self.ecc_bytes or t.param.dtype != dtype:
+                raise ValueError("every tensor of a bucket must share the parameter dtype and the ECC width")
+            if kind != "plain":
+                kernels._check_moment(t.param, t.mom, t.mom_scales, self.quantized, True, "mom")
+            if kind == "adam":
+                kernels._check_moment(t.param, t.var, t.var_scales, self.quantized, False, "var")
         numels = [t.param.numel() for t in tensors]
         p = _native.ptr
         self.table = (FoTensorDesc * self.n_tensors)()

@@ -358,6 +358,55 @@ def test_error_paths():
     assert "FlashOptim Config" in repr(opt3) and "master_bytewidth: 3" in repr(opt3)
 
 
+def test_launch_wrappers_reject_operands_the_kernels_would_overrun():
+    """The kernels see raw addresses only; shapes, dtypes and devices that do not fit are refused on the host, before
+    anything is launched."""
+    from flashoptim_amd import kernels as K
+
+    n = 1000
+    groups = (n + 31) // 32
+    bf = dict(device=DEV, dtype=torch.bfloat16)
+    p, g = torch.zeros(n, **bf), torch.zeros(n, **bf)
+    m, v = torch.zeros(n, device=DEV, dtype=torch.int8), torch.zeros(n, device=DEV, dtype=torch.uint8)
+    sm, sv = torch.zeros(groups, device=DEV, dtype=torch.float16), torch.zeros(groups, device=DEV, dtype=torch.float16)
+    ecc = torch.zeros(n, device=DEV, dtype=torch.int8)
+    hp = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0, decoupled=True, step=1)
+
+    def adam(**over):
+        a = dict(mom=m, mom_scales_f16=sm, var=v, var_scales_f16=sv, param=p, grad=g, errors=ecc)
+        a.update(over)
+        K._fused_adam_step(**a, **hp)
+
+    adam()  # the well-formed call goes through
+    for over, match in [
+        (dict(mom=m[:-1]), "mom must be contiguous with as many elements"),
+        (dict(var=v.to(torch.int8)), "quantised var must be uint8"),
+        (dict(mom_scales_f16=sm[:-1]), "mom scales hold"),
+        (dict(var_scales_f16=sv.float()), "var scales must be a contiguous fp16"),
+        (dict(var_scales_f16=sv.cpu()), "var scales is on cpu"),
+        (dict(errors=ecc[:-1]), "error_bits and param"),
+        (dict(errors=ecc.cpu()), "error_bits is on cpu"),
+        (dict(grad=g.float()), "grad dtype"),
+        (dict(grad=g[:-1]), "same number of elements"),
+    ]:
+        with pytest.raises(ValueError, match=match):
+            adam(**over)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        adam(grad=torch.zeros(2 * n, **bf)[::2])
+    with pytest.raises(ValueError, match="unquantised momentum must have the parameter's dtype"):
+        K._fused_momentum_step(torch.zeros(n, device=DEV), None, p, g, None, 1e-3, 0.9, 1.0, 0.0,
+                               quantize_optim_states=False)
+    with pytest.raises(ValueError, match="out_scales is on cpu"):
+        K.quantize(torch.zeros(n, device=DEV), out_scales=torch.zeros(groups, dtype=torch.float16))
+    with pytest.raises(ValueError, match="in_scales is on cpu"):
+        K.dequantize(m, sm.cpu())
+    with pytest.raises(ValueError, match="error_bits is on cpu"):
+        K.reconstruct_fp32_param(p, ecc.cpu())
+    with pytest.raises(ValueError, match="dst is on cpu"):
+        K.copy_bytes(torch.zeros(n, dtype=torch.int8), m)
+    assert torch.count_nonzero(p) == 0 and torch.count_nonzero(m) == 0   # zero gradients: nothing moved
+
+
 # --------------------------------------------------------------------------------------- state dicts
 
 
