@@ -79,7 +79,7 @@ class FlashAdam(FlashOptimizer):
         return int(param_state["step"].item())
 
     def _kernel_scalars(self, hparams: dict[str, Any], step: Optional[int]) -> dict[str, Any]:
-        lr = hparams["lr"]
+        lr = float(hparams["lr"])  # schedulers may hand over numpy or 0-dim tensor values
         weight_decay = hparams["weight_decay"]
         if self._decoupled:  # the kernel multiplies the weights by 1 - weight_decay (ref:1894-1898)
             weight_decay *= (lr / hparams["initial_lr"]) if self._decouple_lr else lr

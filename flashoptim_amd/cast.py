@@ -80,10 +80,12 @@ def cast_model(
 
     name_of_param = {p: n for n, p in model.named_parameters()}
     name_of_buffer = {b: n for n, b in model.named_buffers()}
-    converted: dict[int, torch.Tensor] = {}  # storage address -> cast tensor, so shared storage is cast once
+    converted: dict[Any, torch.Tensor] = {}  # same memory, same view -> one cast tensor, so tied tensors stay tied
 
     def cast_shared(t: torch.Tensor) -> torch.Tensor:
-        key = t.data.data_ptr()
+        if t.numel() == 0:
+            return t.data.to(dtype=dtype)  # empty tensors all report address 0 without sharing anything
+        key = (t.data.data_ptr(), tuple(t.shape), tuple(t.stride()), t.dtype)
         if key not in converted:
             converted[key] = t.data.to(dtype=dtype)
         return converted[key]

@@ -147,8 +147,7 @@ using namespace fo_host;
 
 // One short-lived workgroup per 4096-element tile (one pass streams better than a persistent grid here); the
 // kernels' tile loop only iterates for tensors beyond 2^31 - 1 tiles.
-unsigned grid_for(int64_t n, int cus) {
-    (void)cus;
+unsigned grid_for(int64_t n) {
     const int64_t tiles = (n + fo::kTileElems - 1) / fo::kTileElems;
     return (unsigned)(tiles < INT32_MAX ? tiles : INT32_MAX);
 }
@@ -164,10 +163,9 @@ int fo_quantize(const void* x, int x_dtype, void* codes, void* scales, int64_t n
     if (n == 0) return 0;  // ref:2485
     if (!x || !codes || !scales) return fail(FO_ERR_INVALID_ARGUMENT, "x, codes and scales must not be NULL");
     if (((uintptr_t)x & (x_dtype == FO_F32 ? 3 : 1)) || ((uintptr_t)scales & 1)) return fail(FO_ERR_INVALID_ARGUMENT, "x or scales not aligned to their element size");
-    const int cus = compute_units();
-    if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
+    if (compute_units() <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
     const fo::CodecFlags f{is_signed ? 1 : 0, do_sqrt ? 1 : 0, softsign ? 1 : 0};
-    const dim3 grid(grid_for(n, cus)), block(fo::kCodecThreads);
+    const dim3 grid(grid_for(n)), block(fo::kCodecThreads);
     hipStream_t s = (hipStream_t)stream;
     switch (x_dtype) {
         case FO_F32: hipLaunchKernelGGL(fo::quantize_kernel<fo::DT_F32>, grid, block, 0, s, x, codes, (uint16_t*)scales, n, f); break;
@@ -183,10 +181,9 @@ int fo_dequantize(const void* codes, const void* scales, float* out, int64_t n, 
     if (n == 0) return 0;  // ref:2533
     if (!codes || !scales || !out) return fail(FO_ERR_INVALID_ARGUMENT, "codes, scales and out must not be NULL");
     if (((uintptr_t)out & 3) || ((uintptr_t)scales & 1)) return fail(FO_ERR_INVALID_ARGUMENT, "out or scales not aligned to their element size");
-    const int cus = compute_units();
-    if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
+    if (compute_units() <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
     const fo::CodecFlags f{is_signed ? 1 : 0, do_sqrt ? 1 : 0, softsign ? 1 : 0};
-    hipLaunchKernelGGL(fo::dequantize_kernel, dim3(grid_for(n, cus)), dim3(fo::kCodecThreads), 0, (hipStream_t)stream, codes,
+    hipLaunchKernelGGL(fo::dequantize_kernel, dim3(grid_for(n)), dim3(fo::kCodecThreads), 0, (hipStream_t)stream, codes,
                        (const uint16_t*)scales, out, n, f);
     return check_hip(hipGetLastError(), "dequantize kernel launch");
 }
@@ -209,9 +206,8 @@ int fo_ecc_join(const void* narrow, int narrow_dtype, const void* ecc, int ecc_b
     if (int rc = validate_ecc_args(narrow, ecc, out, narrow_dtype, ecc_bytes, n)) return rc;
     if (n == 0) return 0;
     if (((uintptr_t)narrow & 1) || ((uintptr_t)out & 3) || (ecc_bytes == 2 && ((uintptr_t)ecc & 1))) return fail(FO_ERR_INVALID_ARGUMENT, "pointer not aligned to its element size");
-    const int cus = compute_units();
-    if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
-    const dim3 grid(grid_for(n, cus)), block(fo::kCodecThreads);
+    if (compute_units() <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
+    const dim3 grid(grid_for(n)), block(fo::kCodecThreads);
     hipStream_t s = (hipStream_t)stream;
     FO_ECC_DISPATCH(ecc_join_kernel, narrow, ecc, out, n)
     return check_hip(hipGetLastError(), "ecc join kernel launch");
@@ -221,9 +217,8 @@ int fo_ecc_split(const float* x, const void* narrow, int narrow_dtype, void* ecc
     if (int rc = validate_ecc_args(x, narrow, ecc, narrow_dtype, ecc_bytes, n)) return rc;
     if (n == 0) return 0;
     if (((uintptr_t)narrow & 1) || ((uintptr_t)x & 3) || (ecc_bytes == 2 && ((uintptr_t)ecc & 1))) return fail(FO_ERR_INVALID_ARGUMENT, "pointer not aligned to its element size");
-    const int cus = compute_units();
-    if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
-    const dim3 grid(grid_for(n, cus)), block(fo::kCodecThreads);
+    if (compute_units() <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
+    const dim3 grid(grid_for(n)), block(fo::kCodecThreads);
     hipStream_t s = (hipStream_t)stream;
     FO_ECC_DISPATCH(ecc_split_kernel, x, narrow, ecc, n)
     return check_hip(hipGetLastError(), "ecc split kernel launch");

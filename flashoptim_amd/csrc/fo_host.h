@@ -26,6 +26,4 @@ int default_tiles_per_chunk();
 // Shared argument check of the multi-tensor entry points: counts, dtype code and table pointers.
 int validate_multi_tables(const void* descs, int64_t n_tensors, const void* chunks, int64_t n_chunks, int dtype);
 
-constexpr int kBlocksPerCu = 8;           // grid cap of the cold-path kernels: blocks per compute unit
-
 }  // namespace fo_host

@@ -59,7 +59,7 @@ class FlashLion(FlashOptimizer):
         return "exp_avg", None
 
     def _kernel_scalars(self, hparams: dict[str, Any], step: Optional[int]) -> dict[str, Any]:
-        lr = hparams["lr"]
+        lr = float(hparams["lr"])  # schedulers may hand over numpy or 0-dim tensor values
         weight_decay = hparams["weight_decay"]  # ref:1290-1294
         weight_decay *= (lr / hparams["initial_lr"]) if self._decouple_lr else lr
         # the kernel's momentum decay is beta2, its update interpolation beta1 (ref:1313-1317)

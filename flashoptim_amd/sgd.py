@@ -67,7 +67,7 @@ class FlashSGD(FlashOptimizer):
         return ("momentum_buffer" if kind == "momentum" else None), None
 
     def _kernel_scalars(self, hparams: dict[str, Any], step: Optional[int]) -> dict[str, Any]:
-        lr = hparams["lr"]
+        lr = float(hparams["lr"])  # schedulers may hand over numpy or 0-dim tensor values
         weight_decay = hparams["weight_decay"]
         if self._decoupled:  # ref:1438-1442
             weight_decay *= (lr / hparams["initial_lr"]) if self._decouple_lr else lr

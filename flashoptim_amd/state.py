@@ -118,7 +118,7 @@ class _MaybeQuantizedTensor:
                 data, signed=self._signed, sqrt=self._sqrt, softsign=self._softsign
             )
         else:
-            self._data = data.to(dtype=self._storage_dtype)
+            self._data = data.to(dtype=self._storage_dtype).contiguous()  # the kernels index it flat
             self._quantized = None
             self._scales = None
 
@@ -175,8 +175,9 @@ class _MaybeQuantizedTensor:
             return
         # torch.optim.Optimizer.load_state_dict has cast both tensors to the parameter dtype on the way in
         self._data = None
-        self._quantized = mine[self._quantized_vals_key(name)].to(dtype=torch.int8 if self._signed else torch.uint8)
-        self._scales = mine[self._quantized_scales_key(name)].to(dtype=torch.float16)
+        codes = mine[self._quantized_vals_key(name)].to(dtype=torch.int8 if self._signed else torch.uint8)
+        self._quantized = codes.contiguous()
+        self._scales = mine[self._quantized_scales_key(name)].to(dtype=torch.float16).contiguous()
 
     @classmethod
     def from_state_dict(

@@ -332,6 +332,22 @@ def test_cast_model_keeps_tied_weights_tied():
     cast_model(m)
     assert a.weight.data_ptr() == b.weight.data_ptr()
 
+    # empty tensors all report address 0 and views of one buffer may start at the same address: neither may be
+    # mistaken for a shared tensor
+    class Odd(nn.Module):
+        def __init__(self):
+            super().__init__()
+            flat = torch.randn(12)
+            self.e1 = nn.Parameter(torch.zeros(0, 4))
+            self.e2 = nn.Parameter(torch.zeros(3, 0))
+            self.v1 = nn.Parameter(flat.view(3, 4))
+            self.v2 = nn.Parameter(flat[:6].view(2, 3))
+
+    m = Odd()
+    cast_model(m)
+    assert [tuple(p.shape) for p in (m.e1, m.e2, m.v1, m.v2)] == [(0, 4), (3, 0), (3, 4), (2, 3)]
+    assert all(p.dtype == torch.bfloat16 for p in m.parameters())
+
 
 # ------------------------------------------------------------------------------------ gradient release
 
