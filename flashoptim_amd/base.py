@@ -77,7 +77,8 @@ class _Bucket:
 @dataclass
 class _GroupCache:
     epoch: int
-    params: list
+    params: list                      # the group's parameter list when the cache was built; keeps `param_ids` unique
+    param_ids: list
     signature: Any
     buckets: list
     idle: list                        # non-empty parameters that had no gradient (or are frozen) when the cache was built
@@ -432,7 +433,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
             if self._check_numerics:
                 each = [self._numerics_needed(p, group["master_bytewidth"]) for b in buckets for p in b.params]
                 needed = max((x for x in each if x is not None), default=None)
-            self._group_cache[index] = _GroupCache(self._plan_epoch, list(group["params"]),
+            self._group_cache[index] = _GroupCache(self._plan_epoch, list(group["params"]), list(map(id, group["params"])),
                                                    self._plan_signature(group), buckets, idle, needed)
         else:
             self._group_cache.pop(index, None)
@@ -446,21 +447,26 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
                 return False
         moved = []
         for b in cache.buckets:
-            ptrs = b.plan.grad_ptrs if b.plan is not None else None
-            for i, p in enumerate(b.params):
+            if b.plan is None:  # single-tensor bucket: launched from the live tensors below
+                for p in b.params:
+                    g = p.grad
+                    if (g is None or not p.requires_grad or g.dtype != b.dtype or g.device != p.device
+                            or not g.is_contiguous()):
+                        return False
+                continue
+            plan, i = b.plan, 0
+            for p, grad_ptr, param_ptr in zip(b.params, plan.grad_ptrs, plan.param_ptrs):
                 g = p.grad
                 if g is None or not p.requires_grad:
                     return False
-                if ptrs is not None:
-                    if p.data_ptr() != b.plan.param_ptrs[i]:
-                        return False  # the parameter's storage was replaced (p.data = ..., module.to(...))
-                    ptr = g.data_ptr()
-                    if ptr != ptrs[i]:
-                        if g.dtype != b.dtype or g.device != p.device or not g.is_contiguous() or g.numel() != p.numel():
-                            return False
-                        moved.append((b.plan, i, ptr))
-                elif g.dtype != b.dtype or g.device != p.device or not g.is_contiguous():
-                    return False
+                if p.data_ptr() != param_ptr:
+                    return False  # the parameter's storage was replaced (p.data = ..., module.to(...))
+                ptr = g.data_ptr()
+                if ptr != grad_ptr:
+                    if g.dtype != b.dtype or g.device != p.device or not g.is_contiguous() or g.numel() != p.numel():
+                        return False
+                    moved.append((plan, i, ptr))
+                i += 1
         for plan, i, ptr in moved:
             plan.set_grad_ptr(i, ptr)
         for b in cache.buckets:
@@ -504,8 +510,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
                 cache is not None
                 and cache.epoch == self._plan_epoch
                 and self._cached_numerics_ok(cache, group)
-                and len(cache.params) == len(group["params"])
-                and all(a is b for a, b in zip(cache.params, group["params"]))
+                and cache.param_ids == list(map(id, group["params"]))
                 and cache.signature == self._plan_signature(group)
                 and self._step_group_fast(cache, group)
             ):
