@@ -977,3 +977,48 @@ def test_deepcopy_of_the_optimizer_is_an_independent_working_optimizer():
         assert torch.equal(a, b)
         assert torch.equal(opt.state[a]["exp_avg"].quantized, twin.state[b]["exp_avg"].quantized)
         assert float(twin.state[b]["step"]) == 4.0
+
+
+@pytest.mark.parametrize("factory,kwargs", [
+    ("FlashAdamW", dict(lr=1e-3, weight_decay=0.01)),
+    ("FlashSGD", dict(lr=1e-2, momentum=0.9, weight_decay=1e-4)),
+])
+def test_scheduler_clipping_and_added_group_match_per_tensor_stepping(factory, kwargs):
+    """The usual furniture of a training loop around step(): a OneCycleLR schedule (moves lr and beta1 / momentum of
+    every group each step), gradient clipping (rewrites the gradients in place) and a parameter group added halfway.
+    step() with its cached plans must stay bit-identical to stepping every tensor on its own."""
+    fo = _fo()
+    shapes = [5000, 33, 4096, 70001]
+    late_shapes = [2049, 64]
+    runs = []
+    for _ in range(2):
+        params, late = _make_params(shapes, torch.bfloat16, 50), _make_params(late_shapes, torch.bfloat16, 51)
+        opt = getattr(fo, factory)(params, **kwargs)
+        sched = torch.optim.lr_scheduler.OneCycleLR(opt, max_lr=kwargs["lr"] * 10, total_steps=12)
+        runs.append((params, late, opt, sched))
+    seen_lrs = set()
+    for it in range(10):
+        for which, (params, late, opt, sched) in enumerate(runs):
+            live = params + (late if it >= 5 else [])
+            if it == 5:  # the schedule keeps its own keys in every group; a late group has to bring them along
+                first = opt.param_groups[0]
+                cycle_keys = [k for k in first if k.startswith(("max_", "min_", "base_", "initial_"))]
+                opt.add_param_group(dict(params=late, **{k: first[k] for k in cycle_keys}))
+            _set_grads(live, 500 + it, scale=1e-2)
+            torch.nn.utils.clip_grad_norm_(live, 0.05)
+            if which == 0:
+                opt.step()
+            else:
+                for p in live:
+                    opt.step_param(p)
+            with warnings.catch_warnings():
+                warnings.simplefilter("ignore")  # the per-tensor run never calls step(), which the scheduler remarks on
+                sched.step()
+            seen_lrs.add(opt.param_groups[0]["lr"])
+    assert len(seen_lrs) == 10, "the schedule should have changed lr every step"
+    (pa, la, oa, _), (pb, lb, ob, _) = runs
+    for a, b in zip(pa + la, pb + lb):
+        assert torch.equal(a, b)
+        sa, sb = _state_tensors(oa, a), _state_tensors(ob, b)
+        for k in sa:
+            assert parity.bits_equal(sa[k], sb[k]), k
