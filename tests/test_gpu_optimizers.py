@@ -1022,3 +1022,52 @@ def test_scheduler_clipping_and_added_group_match_per_tensor_stepping(factory, k
         sa, sb = _state_tensors(oa, a), _state_tensors(ob, b)
         for k in sa:
             assert parity.bits_equal(sa[k], sb[k]), k
+
+
+@pytest.mark.parametrize("factory,kwargs", [
+    ("FlashLion", dict(lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1)),
+    ("FlashSGDW", dict(lr=1e-2, momentum=0.9, weight_decay=1e-4)),
+])
+def test_step_of_the_counter_free_optimizers_can_be_captured_in_a_graph(factory, kwargs):
+    """Lion and SGD pass no step counter to their kernels, so once the launch plan is cached step() is nothing but
+    kernel launches on the current stream and can be recorded into a HIP graph over static gradient buffers.  Every
+    replay is checked against an eagerly stepped twin, with eager work and synchronisations in between."""
+    fo = _fo()
+    shapes = [5000, 33, 4096, 70001]
+    pa, pb = _make_params(shapes, torch.bfloat16, 60), _make_params(shapes, torch.bfloat16, 60)
+    oa, ob = getattr(fo, factory)(pa, **kwargs), getattr(fo, factory)(pb, **kwargs)
+    _set_grads(pa, 600)
+    static_grads = [p.grad for p in pa]
+
+    def feed(seed):
+        _set_grads(pb, seed)
+        for g, p in zip(static_grads, pb):
+            g.copy_(p.grad)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for it in range(2):               # builds the states and the cached plan outside the graph
+            feed(600 + it)
+            oa.step()
+            ob.step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    feed(602)
+    with torch.cuda.graph(graph):
+        oa.step()
+    graph.replay()
+    ob.step()
+    for it in range(3, 7):
+        feed(600 + it)
+        torch.cuda.synchronize()
+        graph.replay()
+        ob.step()
+        torch.cuda.synchronize()
+        for a, b in zip(pa, pb):
+            assert torch.equal(a, b), (it, a.numel())
+    for a, b in zip(pa, pb):
+        sa, sb = _state_tensors(oa, a), _state_tensors(ob, b)
+        for k in sa:
+            assert parity.bits_equal(sa[k], sb[k]), k
