@@ -64,6 +64,10 @@ class FlashAdam(FlashOptimizer):
             # a CPU fp32 scalar like torch's own optimizers checkpoint it; reading it never syncs the device
             state["step"] = torch.tensor(0, dtype=torch.float32, device="cpu")
 
+    # the kernels take the step number by value (ref:2368-2369): a replayed graph would repeat one step's bias
+    # correction while the CPU counters stand still
+    _step_number_by_value = True
+
     def _min_step_size_relative_to_lr(self) -> float:
         # |m| / sqrt(v) has no positive lower bound; assume updates routinely shrink to a tenth of lr
         return 0.1

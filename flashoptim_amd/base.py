@@ -223,6 +223,16 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
     def _min_step_size_relative_to_lr(self) -> float:
         return 1.0  # sign-based updates (Lion) move every weight by exactly lr
 
+    # True for optimizers whose kernels receive a per-parameter step number as a host value
+    _step_number_by_value = False
+
+    def _refuse_graph_capture(self) -> None:
+        if self._step_number_by_value and torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(
+                f"{type(self).__name__} cannot be stepped while a HIP graph is being recorded: its bias correction "
+                "depends on the step number, which the kernels receive as a host value."
+            )
+
     # ------------------------------------------------------------------------------ sharded-tensor shims
     @staticmethod
     def _get_tensor_for_stats(tensor: torch.Tensor) -> torch.Tensor:
@@ -379,6 +389,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         """
         if group is None:
             group = self._find_group(p)
+        self._refuse_graph_capture()
         self._plan_epoch += 1  # counters move outside step(): cached bucket state is stale
         plan = self._plan_param(p, group)
         if plan is not None:
@@ -500,6 +511,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
                 stacklevel=2,
             )
             return None
+        self._refuse_graph_capture()
         loss = None
         if closure is not None:
             with torch.enable_grad():

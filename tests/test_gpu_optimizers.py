@@ -1071,3 +1071,30 @@ def test_step_of_the_counter_free_optimizers_can_be_captured_in_a_graph(factory,
         sa, sb = _state_tensors(oa, a), _state_tensors(ob, b)
         for k in sa:
             assert parity.bits_equal(sa[k], sb[k]), k
+
+
+def test_adam_step_refuses_graph_capture():
+    """Adam's bias correction takes the step number by value: a replayed graph would repeat it, so capture raises
+    instead of going quietly wrong, and leaves the optimizer usable."""
+    fo = _fo()
+    params = _make_params([4096, 33], torch.bfloat16, 61)
+    opt = fo.FlashAdamW(params, lr=1e-3)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for it in range(2):
+            _set_grads(params, 610 + it)
+            opt.step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")   # torch remarks that the abandoned graph is empty
+        with pytest.raises(RuntimeError, match="while a HIP graph is being recorded"):
+            with torch.cuda.graph(graph):
+                opt.step()
+    torch.cuda.synchronize()
+    before = params[0].clone()
+    opt.step()
+    assert not torch.equal(params[0], before)
+    assert all(float(opt.state[p]["step"]) == 3.0 for p in params), "the refused step must not count"
