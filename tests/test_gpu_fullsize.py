@@ -166,3 +166,62 @@ def test_ragged_4096_tensor_launch_equals_per_tensor_launches():
         assert torch.equal(sa["error_bits"], sb["error_bits"])
         assert torch.equal(sa["exp_avg"].quantized, sb["exp_avg"].quantized)
         assert parity.bits_equal(sa["exp_avg"].scales, sb["exp_avg"].scales)
+
+
+def _llama3_8b_lengths():
+    h, ffn, kv, vocab = 4096, 14336, 1024, 128256
+    lens = [vocab * h]
+    for _ in range(32):
+        lens += [h * h, kv * h, kv * h, h * h, ffn * h, ffn * h, h * ffn, h, h]
+    return lens + [h, vocab * h]
+
+
+@pytest.mark.parametrize("mwb", [32, 24])
+def test_llama8b_multi_tensor_launch_equals_per_tensor_launches(mwb):
+    """The 8B configuration at full size (291 bf16 tensors of Llama-3-8B's shapes, 8 030 261 248 elements, FlashAdamW
+    with 32-bit and with 24-bit master weights): one multi-tensor launch per step is bit-identical to 291
+    single-tensor launches, and every tensor moved."""
+    import gc
+    import warnings
+
+    import flashoptim_amd as fo
+
+    lens = _llama3_8b_lengths()
+    assert len(lens) == 291 and sum(lens) == 8_030_261_248
+    dg = torch.Generator(device=DEV).manual_seed(11)
+    pa = []
+    for n in lens:
+        p = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+        for i in range(0, n, 1 << 27):
+            m = min(1 << 27, n - i)
+            p[i:i + m] = (torch.randn(m, generator=dg, device=DEV) * 0.02).to(torch.bfloat16)
+        pa.append(torch.nn.Parameter(p))
+    pb = [torch.nn.Parameter(p.detach().clone()) for p in pa]
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        oa = fo.FlashAdamW(pa, lr=1e-3, weight_decay=0.01, master_weight_bits=mwb)
+        ob = fo.FlashAdamW(pb, lr=1e-3, weight_decay=0.01, master_weight_bits=mwb)
+    for it in range(2):
+        for a, b in zip(pa, pb):
+            if a.grad is None:
+                a.grad = torch.empty_like(a)
+            for i in range(0, a.numel(), 1 << 27):
+                m = min(1 << 27, a.numel() - i)
+                a.grad[i:i + m] = (torch.randn(m, generator=dg, device=DEV) * 1e-3).to(torch.bfloat16)
+            b.grad = a.grad          # read-only for the kernels: both optimizers may share it
+        oa.step()
+        for p in pb:
+            ob.step_param(p)
+    torch.cuda.synchronize()
+    for a, b in zip(pa, pb):
+        assert torch.equal(a, b)
+        sa, sb = oa.state[a], ob.state[b]
+        assert sa["error_bits"].dtype == (torch.int16 if mwb == 32 else torch.int8)
+        assert torch.equal(sa["error_bits"], sb["error_bits"])
+        for name in ("exp_avg", "exp_avg_sq"):
+            assert torch.equal(sa[name].quantized, sb[name].quantized)
+            assert parity.bits_equal(sa[name].scales, sb[name].scales)
+        assert bool(sa["exp_avg"].quantized.any()) and float(sa["step"]) == 2.0
+    del oa, ob, pa, pb
+    gc.collect()
+    torch.cuda.empty_cache()
