@@ -170,3 +170,119 @@ def test_decouple_lr_variants_match_their_textbook_forms(kind):
         assert np.mean(np.abs(got - ref) > 1e-6) < 2e-3
     else:
         np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-7)
+
+
+# ---------------------------------------------------------------------------------- a small language model
+
+
+class _Block(nn.Module):
+    def __init__(self, d, heads):
+        super().__init__()
+        self.heads = heads
+        self.ln1, self.ln2 = nn.LayerNorm(d), nn.LayerNorm(d)
+        self.qkv, self.proj = nn.Linear(d, 3 * d), nn.Linear(d, d)
+        self.up, self.down = nn.Linear(d, 4 * d), nn.Linear(4 * d, d)
+
+    def forward(self, x, mask):
+        b, t, d = x.shape
+        q, k, v = self.qkv(self.ln1(x)).view(b, t, 3, self.heads, d // self.heads).permute(2, 0, 3, 1, 4)
+        att = (q @ k.transpose(-1, -2)) / (d // self.heads) ** 0.5 + mask
+        x = x + self.proj((att.softmax(-1) @ v).transpose(1, 2).reshape(b, t, d))
+        return x + self.down(torch.nn.functional.gelu(self.up(self.ln2(x))))
+
+
+class _TinyLM(nn.Module):
+    """Two pre-norm transformer blocks over a tied embedding / output matrix: 1-D norm weights, biases, 2-D and
+    tied parameters in one model, i.e. every parameter flavour the optimizers meet in a language model."""
+
+    def __init__(self, vocab=128, d=64, heads=4, seq=32):
+        super().__init__()
+        self.embed = nn.Embedding(vocab, d)
+        self.pos = nn.Parameter(torch.zeros(seq, d))
+        self.blocks = nn.ModuleList([_Block(d, heads) for _ in range(2)])
+        self.norm = nn.LayerNorm(d)
+        self.head = nn.Linear(d, vocab, bias=False)
+        self.head.weight = self.embed.weight
+        self.register_buffer("mask", torch.full((seq, seq), float("-inf")).triu(1))
+
+    def forward(self, idx):
+        x = self.embed(idx) + self.pos
+        for blk in self.blocks:
+            x = blk(x, self.mask.to(x.dtype))
+        return self.head(self.norm(x))
+
+
+def _lm_batch(step, vocab=128, seq=32, batch=16):
+    """Sequences that count upwards modulo the vocabulary in strides of 1..4 from random starts: the next token
+    follows from the previous two."""
+    g = torch.Generator().manual_seed(1000 + step)
+    start = torch.randint(0, vocab, (batch, 1), generator=g)
+    stride = torch.randint(1, 5, (batch, 1), generator=g)
+    tokens = (start + stride * torch.arange(seq + 1)) % vocab
+    return tokens[:, :-1].to(DEV), tokens[:, 1:].to(DEV)
+
+
+def _lm_loss(model, step):
+    x, y = _lm_batch(step)
+    return nn.functional.cross_entropy(model(x).float().flatten(0, 1), y.flatten())
+
+
+def _lm_run(make_opt, steps, bf16, release=False, resume_at=None):
+    fo = _fo()
+    torch.manual_seed(0)
+    model = _TinyLM().to(DEV)
+    if bf16:
+        fo.cast_model(model)
+    opt = make_opt(model.parameters())
+    handle = fo.enable_gradient_release(model, opt) if release else None
+    losses = []
+    for step in range(steps):
+        if resume_at is not None and step == resume_at:    # checkpoint, rebuild everything, carry on
+            blob = (copy.deepcopy(model.state_dict()), copy.deepcopy(opt.state_dict()))
+            torch.manual_seed(1)
+            model = _TinyLM().to(DEV)
+            if bf16:
+                fo.cast_model(model)
+            model.load_state_dict(blob[0])
+            opt = make_opt(model.parameters())
+            opt.load_state_dict(blob[1])
+        loss = _lm_loss(model, step)
+        loss.backward()
+        if not release:
+            opt.step()
+            opt.zero_grad()
+        losses.append(loss.item())
+    if handle is not None:
+        handle.remove()
+    return np.array(losses), model, opt
+
+
+def test_tiny_language_model_trains_like_fp32_adamw():
+    """cast_model + FlashAdamW (bf16 weights, 24-bit masters, 8-bit moments) on a small transformer against an fp32
+    model under torch.optim.AdamW: same data, same initialisation, 300 steps.  The loss must fall as far and follow
+    the same curve; with gradient release the run is the same computation launched from the hooks; a compressed
+    checkpoint taken halfway resumes onto the same curve."""
+    fo = _fo()
+    hp = dict(lr=3e-3, betas=(0.9, 0.99), weight_decay=0.01)
+    steps = 300
+    ref, _, _ = _lm_run(lambda ps: torch.optim.AdamW(ps, **hp), steps, bf16=False)
+    flash = lambda ps: fo.FlashAdamW(ps, master_weight_bits=24, compress_state_dict=True, **hp)  # noqa: E731
+    got, model, opt = _lm_run(flash, steps, bf16=True)
+    assert ref[0] > 4.5 and ref[-20:].mean() < 0.5, "the fp32 run should have learned the task"
+    assert abs(got[-20:].mean() - ref[-20:].mean()) < 0.15 * ref[-20:].mean(), (got[-20:].mean(), ref[-20:].mean())
+    smooth = lambda a: np.convolve(a, np.ones(10) / 10, mode="valid")  # noqa: E731
+    assert np.corrcoef(smooth(got), smooth(ref))[0, 1] > 0.999        # measured 0.99997
+    # every parameter flavour got its state; the tied matrix has one
+    assert len(opt.state) == len(list(model.parameters())) and model.head.weight is model.embed.weight
+    assert all(s["error_bits"].dtype == torch.int8 and s["exp_avg"].is_quantized() for s in opt.state.values())
+
+    released, _, _ = _lm_run(flash, steps, bf16=True, release=True)
+    assert abs(released[-20:].mean() - got[-20:].mean()) < 0.01 and np.corrcoef(smooth(released), smooth(got))[0, 1] > 0.9999
+
+    resumed, _, _ = _lm_run(flash, steps, bf16=True, resume_at=150)
+    assert np.array_equal(resumed[:150], got[:150])
+    assert np.allclose(resumed[150:], got[150:], rtol=0.05, atol=0.02), np.abs(resumed[150:] - got[150:]).max()
+    print(f"tiny LM, mean loss of the last 20 steps: fp32 AdamW {ref[-20:].mean():.4f}, FlashAdamW {got[-20:].mean():.4f}, "
+          f"with gradient release {released[-20:].mean():.4f}, resumed {resumed[-20:].mean():.4f}; "
+          f"largest loss difference after the resume {np.abs(resumed[150:] - got[150:]).max():.4f}; "
+          f"curve correlation with fp32 {np.corrcoef(smooth(got), smooth(ref))[0, 1]:.5f}")
