@@ -355,3 +355,20 @@ def test_cast_model_keeps_tied_weights_tied():
 def test_gradient_release_rejects_grad_scaler_before_anything_else():
     with pytest.raises(NotImplementedError, match="GradScaler"):
         enable_gradient_release(nn.Linear(2, 2), optimizer=None, grad_scaler=object())
+
+
+def test_packaging_declares_the_reference_entry_points():
+    """llm-foundry discovers optimizers through the `llmfoundry_optimizers` entry-point group; the names are the
+    reference's (/root/reference/pyproject.toml:47-52) and every target resolves to a class of this package."""
+    import importlib
+    import os
+
+    import tomli
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(os.path.join(root, "pyproject.toml"), "rb") as f:
+        points = tomli.load(f)["project"]["entry-points"]["llmfoundry_optimizers"]
+    assert sorted(points) == ["flash_adam", "flash_adam_w", "flash_lion", "flash_sgd", "flash_sgd_w"]
+    for target in points.values():
+        module, _, name = target.partition(":")
+        assert issubclass(getattr(importlib.import_module(module), name), torch.optim.Optimizer)
