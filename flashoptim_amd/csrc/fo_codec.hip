@@ -11,7 +11,7 @@
 
 namespace fo {
 
-constexpr int kCodecThreads = 256;
+constexpr int kCodecThreads = 64;   // one wavefront per workgroup, like the step kernels
 
 struct CodecFlags {
     int is_signed, do_sqrt, softsign;
@@ -47,27 +47,45 @@ __device__ __forceinline__ void quantize_lane(const void* x, void* codes, uint16
     if ((FAST || first < n) && (threadIdx.x & (32 / EPL - 1)) == 0) store_scale(scales, first >> 5, f32_to_f16_bits(am));   // ref:2675-2676
 }
 
+// Value of code byte b before the group scale: q / IN_MAX, then y / (2 - |y|) when the softsign companding is on
+// (ref:2591-2597), each operation correctly rounded.  Evaluated by the compiler, one table per flag combination;
+// a lookup replaces two IEEE divisions per element.
+template <bool SIGNED, bool SOFTSIGN> struct CodeTable {
+    float v[256];
+    constexpr CodeTable() : v() {
+        for (int b = 0; b < 256; ++b) {
+            const int q = (SIGNED && b >= 128) ? b - 256 : b;
+            const float t = (float)q / (SIGNED ? 127.0f : 255.0f);
+            const float a = t < 0.0f ? -t : t;
+            v[b] = SOFTSIGN ? t / (2.0f - a) : t;
+        }
+    }
+};
+__device__ const CodeTable<false, false> kCodeTableU = CodeTable<false, false>();
+__device__ const CodeTable<false, true> kCodeTableUS = CodeTable<false, true>();
+__device__ const CodeTable<true, false> kCodeTableS = CodeTable<true, false>();
+__device__ const CodeTable<true, true> kCodeTableSS = CodeTable<true, true>();
+
 // ref:2541-2607 _triton_dequantize_kernel
 template <bool FAST>
-__device__ __forceinline__ void dequantize_lane(const void* codes, const uint16_t* scales, float* out, int64_t first, int64_t n, CodecFlags f) {
-    constexpr int EPL = 4;
-    Pack<1, EPL> craw;
-    load_lane<1, EPL, FAST>(craw, codes, first, n);
-    float scale = 1.0f;                                                     // ref:2577-2582 masked scales read 1.0
-    if (FAST || first < n) scale = f16_bits_to_f32(scales[first >> 5]);
-    const float in_max = f.is_signed ? 127.0f : 255.0f;
-    Pack<4, EPL> o;
+__device__ __forceinline__ void dequantize_load(const void* codes, const uint16_t* scales, int64_t first, int64_t n,
+                                                Pack<1, 4>& craw, uint16_t& scale_bits) {
+    load_lane<1, 4, FAST>(craw, codes, first, n);
+    scale_bits = 0x3c00;                                                    // ref:2577-2582 masked scales read 1.0
+    if (FAST || first < n) scale_bits = scales[first >> 5];
+}
+template <bool FAST>
+__device__ __forceinline__ void dequantize_finish(const Pack<1, 4>& craw, uint16_t scale_bits, const float* lut, float* out,
+                                                  int64_t first, int64_t n, CodecFlags f) {
+    const float scale = f16_bits_to_f32(scale_bits);
+    Pack<4, 4> o;
 #pragma unroll
-    for (int k = 0; k < EPL; ++k) {
-        const u32 b = byte_of<EPL>(craw, k);
-        const float q = f.is_signed ? (float)(int8_t)b : (float)b;
-        const float t = div_rn(q, in_max);                                  // ref:2591
-        const float nrm = f.softsign ? div_rn(t, 2.0f - fabsf(t)) : t;      // ref:2594-2597
-        float xv = nrm * scale;                                             // ref:2600
+    for (int k = 0; k < 4; ++k) {
+        float xv = lut[byte_of<4>(craw, k)] * scale;                        // ref:2591-2600
         if (f.do_sqrt) xv = xv * xv;                                        // ref:2603-2604
         o.w[k] = as_u32(xv);
     }
-    store_lane<4, EPL, FAST>(o, out, first, n);
+    store_lane<4, 4, FAST>(o, out, first, n);
 }
 
 // ref:2779-2803 _reconstruct_fp32_kernel
@@ -100,44 +118,73 @@ __device__ __forceinline__ void ecc_split_lane(const float* x, const void* narro
     store_lane<ECCB, EPL, FAST>(eout, ecc, first, n);
 }
 
-// Tile loop shared by the four kernels: blocks stride over 4096-element tiles, wavefronts over the tile's
-// sub-tiles of 64 x EPL elements; `first` is the lane's first element.
-#define FO_TILE_LOOP(N, EPL_, ALIGNED, CALL_FAST, CALL_SLOW)                                      \
+// Work loop shared by the four kernels, in the step kernels' geometry: a workgroup is one wavefront and takes one
+// span of 64 x EPL elements (it only iterates for tensors beyond 2^31 - 1 spans); `first` is the lane's first element.
+#define FO_SPAN_LOOP(N, EPL_, ALIGNED, CALL_FAST, CALL_SLOW)                                      \
     {                                                                                             \
-        constexpr int kSub_ = 64 * (EPL_);                                                        \
-        const int lane_ = threadIdx.x & 63, wave_ = threadIdx.x >> 6;                             \
-        const int64_t n_tiles_ = ((N) + kTileElems - 1) / kTileElems;                             \
-        for (int64_t tile_ = blockIdx.x; tile_ < n_tiles_; tile_ += gridDim.x) {                  \
-            const int64_t base_ = tile_ * (int64_t)kTileElems;                                    \
-            const bool fast_ = (ALIGNED) && base_ + kTileElems <= (N);                            \
-            for (int s_ = wave_; s_ < kTileElems / kSub_; s_ += kCodecThreads / 64) {             \
-                const int64_t first = base_ + s_ * kSub_ + lane_ * (EPL_);                        \
-                if (fast_) { CALL_FAST; } else { CALL_SLOW; }                                     \
-            }                                                                                     \
+        constexpr int64_t kSpan_ = 64 * (EPL_);                                                   \
+        const int64_t n_spans_ = ((N) + kSpan_ - 1) / kSpan_;                                     \
+        for (int64_t span_ = blockIdx.x; span_ < n_spans_; span_ += gridDim.x) {                  \
+            const int64_t first = span_ * kSpan_ + (int64_t)threadIdx.x * (EPL_);                 \
+            if ((ALIGNED) && (span_ + 1) * kSpan_ <= (N)) { CALL_FAST; } else { CALL_SLOW; }      \
         }                                                                                         \
     }
 
 template <int XDT>
 __global__ __launch_bounds__(kCodecThreads) void quantize_kernel(const void* x, void* codes, uint16_t* scales, int64_t n, CodecFlags f) {
     const bool aligned = ((((uintptr_t)x) | ((uintptr_t)codes)) & 15u) == 0;
-    FO_TILE_LOOP(n, DTypeInfo<XDT>::epl, aligned, (quantize_lane<XDT, true>(x, codes, scales, first, n, f)), (quantize_lane<XDT, false>(x, codes, scales, first, n, f)))
+    FO_SPAN_LOOP(n, DTypeInfo<XDT>::epl, aligned, (quantize_lane<XDT, true>(x, codes, scales, first, n, f)), (quantize_lane<XDT, false>(x, codes, scales, first, n, f)))
 }
 
+// A workgroup (one wavefront) takes kDequantSpans neighbouring spans of 256 elements, so that the 1 KiB table it
+// copies to LDS serves more than one span (4 spans: 5.6 TB/s, 1 span: 4.7; reading the table through the vector
+// cache instead: 3.5); all code loads are issued before the table is committed.  Four of every five bytes are
+// written, and write-only streams reach 5.7-6.0 TB/s on this part.
+constexpr int kDequantSpans = 4;
 __global__ __launch_bounds__(kCodecThreads) void dequantize_kernel(const void* codes, const uint16_t* scales, float* out, int64_t n, CodecFlags f) {
+    constexpr int kSpans = kDequantSpans;
+    constexpr int64_t kSpan = 64 * 4;
     const bool aligned = ((((uintptr_t)out) | ((uintptr_t)codes)) & 15u) == 0;
-    FO_TILE_LOOP(n, 4, aligned, (dequantize_lane<true>(codes, scales, out, first, n, f)), (dequantize_lane<false>(codes, scales, out, first, n, f)))
+    const float* table = f.is_signed ? (f.softsign ? kCodeTableSS.v : kCodeTableS.v) : (f.softsign ? kCodeTableUS.v : kCodeTableU.v);
+    __shared__ __align__(16) float lut[256];
+    const u32x4 frag = *reinterpret_cast<const u32x4*>(table + 4 * threadIdx.x);
+    bool committed = false;
+    const int64_t n_blocks = (n + kSpan * kSpans - 1) / (kSpan * kSpans);
+    for (int64_t blk = blockIdx.x; blk < n_blocks; blk += gridDim.x) {
+        const int64_t base = blk * kSpan * kSpans;
+        const bool fast = aligned && base + kSpan * kSpans <= n;
+        Pack<1, 4> craw[kSpans];
+        uint16_t scale_bits[kSpans];
+#pragma unroll
+        for (int i = 0; i < kSpans; ++i) {
+            const int64_t first = base + i * kSpan + (int64_t)threadIdx.x * 4;
+            if (fast) dequantize_load<true>(codes, scales, first, n, craw[i], scale_bits[i]);
+            else dequantize_load<false>(codes, scales, first, n, craw[i], scale_bits[i]);
+        }
+        if (!committed) {
+            *reinterpret_cast<u32x4*>(lut + 4 * threadIdx.x) = frag;
+            __syncthreads();  // one wavefront: no hardware barrier is needed, the compiler drops it
+            committed = true;
+        }
+#pragma unroll
+        for (int i = 0; i < kSpans; ++i) {
+            const int64_t first = base + i * kSpan + (int64_t)threadIdx.x * 4;
+            if (fast) dequantize_finish<true>(craw[i], scale_bits[i], lut, out, first, n, f);
+            else dequantize_finish<false>(craw[i], scale_bits[i], lut, out, first, n, f);
+        }
+    }
 }
 
 template <int DT, int ECCB>
 __global__ __launch_bounds__(kCodecThreads) void ecc_join_kernel(const void* narrow, const void* ecc, float* out, int64_t n) {
     const bool aligned = ((((uintptr_t)narrow) | ((uintptr_t)ecc) | ((uintptr_t)out)) & 15u) == 0;
-    FO_TILE_LOOP(n, 4, aligned, (ecc_join_lane<DT, ECCB, true>(narrow, ecc, out, first, n)), (ecc_join_lane<DT, ECCB, false>(narrow, ecc, out, first, n)))
+    FO_SPAN_LOOP(n, 4, aligned, (ecc_join_lane<DT, ECCB, true>(narrow, ecc, out, first, n)), (ecc_join_lane<DT, ECCB, false>(narrow, ecc, out, first, n)))
 }
 
 template <int DT, int ECCB>
 __global__ __launch_bounds__(kCodecThreads) void ecc_split_kernel(const float* x, const void* narrow, void* ecc, int64_t n) {
     const bool aligned = ((((uintptr_t)narrow) | ((uintptr_t)ecc) | ((uintptr_t)x)) & 15u) == 0;
-    FO_TILE_LOOP(n, 4, aligned, (ecc_split_lane<DT, ECCB, true>(x, narrow, ecc, first, n)), (ecc_split_lane<DT, ECCB, false>(x, narrow, ecc, first, n)))
+    FO_SPAN_LOOP(n, 4, aligned, (ecc_split_lane<DT, ECCB, true>(x, narrow, ecc, first, n)), (ecc_split_lane<DT, ECCB, false>(x, narrow, ecc, first, n)))
 }
 
 }  // namespace fo
@@ -145,11 +192,10 @@ __global__ __launch_bounds__(kCodecThreads) void ecc_split_kernel(const float* x
 namespace {
 using namespace fo_host;
 
-// One short-lived workgroup per 4096-element tile (one pass streams better than a persistent grid here); the
-// kernels' tile loop only iterates for tensors beyond 2^31 - 1 tiles.
-unsigned grid_for(int64_t n) {
-    const int64_t tiles = (n + fo::kTileElems - 1) / fo::kTileElems;
-    return (unsigned)(tiles < INT32_MAX ? tiles : INT32_MAX);
+// One short-lived workgroup per span of 64 x EPL elements (one pass streams better than a persistent grid here).
+unsigned grid_for(int64_t n, int epl) {
+    const int64_t spans = (n + 64 * epl - 1) / (64 * epl);
+    return (unsigned)(spans < INT32_MAX ? spans : INT32_MAX);
 }
 
 }  // namespace
@@ -165,7 +211,7 @@ int fo_quantize(const void* x, int x_dtype, void* codes, void* scales, int64_t n
     if (((uintptr_t)x & (x_dtype == FO_F32 ? 3 : 1)) || ((uintptr_t)scales & 1)) return fail(FO_ERR_INVALID_ARGUMENT, "x or scales not aligned to their element size");
     if (compute_units() <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
     const fo::CodecFlags f{is_signed ? 1 : 0, do_sqrt ? 1 : 0, softsign ? 1 : 0};
-    const dim3 grid(grid_for(n)), block(fo::kCodecThreads);
+    const dim3 grid(grid_for(n, x_dtype == FO_F32 ? 4 : 8)), block(fo::kCodecThreads);
     hipStream_t s = (hipStream_t)stream;
     switch (x_dtype) {
         case FO_F32: hipLaunchKernelGGL(fo::quantize_kernel<fo::DT_F32>, grid, block, 0, s, x, codes, (uint16_t*)scales, n, f); break;
@@ -183,7 +229,7 @@ int fo_dequantize(const void* codes, const void* scales, float* out, int64_t n, 
     if (((uintptr_t)out & 3) || ((uintptr_t)scales & 1)) return fail(FO_ERR_INVALID_ARGUMENT, "out or scales not aligned to their element size");
     if (compute_units() <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
     const fo::CodecFlags f{is_signed ? 1 : 0, do_sqrt ? 1 : 0, softsign ? 1 : 0};
-    hipLaunchKernelGGL(fo::dequantize_kernel, dim3(grid_for(n)), dim3(fo::kCodecThreads), 0, (hipStream_t)stream, codes,
+    hipLaunchKernelGGL(fo::dequantize_kernel, dim3(grid_for(n, 4 * fo::kDequantSpans)), dim3(fo::kCodecThreads), 0, (hipStream_t)stream, codes,
                        (const uint16_t*)scales, out, n, f);
     return check_hip(hipGetLastError(), "dequantize kernel launch");
 }
@@ -207,7 +253,7 @@ int fo_ecc_join(const void* narrow, int narrow_dtype, const void* ecc, int ecc_b
     if (n == 0) return 0;
     if (((uintptr_t)narrow & 1) || ((uintptr_t)out & 3) || (ecc_bytes == 2 && ((uintptr_t)ecc & 1))) return fail(FO_ERR_INVALID_ARGUMENT, "pointer not aligned to its element size");
     if (compute_units() <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
-    const dim3 grid(grid_for(n)), block(fo::kCodecThreads);
+    const dim3 grid(grid_for(n, 4)), block(fo::kCodecThreads);
     hipStream_t s = (hipStream_t)stream;
     FO_ECC_DISPATCH(ecc_join_kernel, narrow, ecc, out, n)
     return check_hip(hipGetLastError(), "ecc join kernel launch");
@@ -218,7 +264,7 @@ int fo_ecc_split(const float* x, const void* narrow, int narrow_dtype, void* ecc
     if (n == 0) return 0;
     if (((uintptr_t)narrow & 1) || ((uintptr_t)x & 3) || (ecc_bytes == 2 && ((uintptr_t)ecc & 1))) return fail(FO_ERR_INVALID_ARGUMENT, "pointer not aligned to its element size");
     if (compute_units() <= 0) return fail(FO_ERR_NO_DEVICE, "no HIP device");
-    const dim3 grid(grid_for(n)), block(fo::kCodecThreads);
+    const dim3 grid(grid_for(n, 4)), block(fo::kCodecThreads);
     hipStream_t s = (hipStream_t)stream;
     FO_ECC_DISPATCH(ecc_split_kernel, x, narrow, ecc, n)
     return check_hip(hipGetLastError(), "ecc split kernel launch");
