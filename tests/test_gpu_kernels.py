@@ -421,8 +421,8 @@ def test_randomised_configurations_match_oracle():
 
 
 def test_the_binding_shown_in_the_integration_notes_runs():
-    """The ctypes stub printed in INTEGRATION.md (what a maintainer of the reference would add) is executed as
-    written, against the built library, and gives the same bits as this package's own binding."""
+    """The ctypes stub that the integration notes print (what a maintainer of the reference would add) is executed
+    as written, against the built library, and gives the same bits as this package's own binding."""
     import os
     import re
 
