@@ -125,8 +125,9 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED> struct AdamOp {
     using Hyper = AdamHyper;
     static constexpr bool kNeedsLut = QUANT;
     // measured on MI355X with the 8B-parameter step: 14-15 resident workgroups per compute unit for 2-byte
-    // parameters (3.6-4.5 KiB of loads per wavefront), 16-20 for fp32 parameters (2.5 KiB)
-    static constexpr int kLdsBytes = DT == DT_F32 ? 9216 : 11008;
+    // parameters with no or a 1-byte ECC (3.6-4.1 KiB of loads per wavefront), 13 with a 2-byte ECC (4.6 KiB),
+    // 16-20 for fp32 parameters (2.5 KiB)
+    static constexpr int kLdsBytes = DT == DT_F32 ? 9216 : (ECCB == 2 ? 12288 : 11008);
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, int64_t first, Raw& r) {
