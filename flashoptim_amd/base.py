@@ -82,6 +82,7 @@ class _GroupCache:
     signature: Any
     buckets: list
     idle: list                        # non-empty parameters that had no gradient (or are frozen) when the cache was built
+    state_len: int                    # len(optimizer.state) then: a cleared or pruned state dict invalidates the cache
     # check_numerics: log2 of the coarsest weight resolution over the group's parameters (None: nothing to check)
     numerics_needed: Optional[float] = None
 
@@ -445,7 +446,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
                 each = [self._numerics_needed(p, group["master_bytewidth"]) for b in buckets for p in b.params]
                 needed = max((x for x in each if x is not None), default=None)
             self._group_cache[index] = _GroupCache(self._plan_epoch, list(group["params"]), list(map(id, group["params"])),
-                                                   self._plan_signature(group), buckets, idle, needed)
+                                                   self._plan_signature(group), buckets, idle, len(self.state), needed)
         else:
             self._group_cache.pop(index, None)
 
@@ -521,6 +522,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
             if (
                 cache is not None
                 and cache.epoch == self._plan_epoch
+                and cache.state_len == len(self.state)
                 and self._cached_numerics_ok(cache, group)
                 and cache.param_ids == list(map(id, group["params"]))
                 and cache.signature == self._plan_signature(group)

@@ -1098,3 +1098,33 @@ def test_adam_step_refuses_graph_capture():
     opt.step()
     assert not torch.equal(params[0], before)
     assert all(float(opt.state[p]["step"]) == 3.0 for p in params), "the refused step must not count"
+
+
+def test_clearing_the_optimizer_state_restarts_the_moments():
+    """`optimizer.state.clear()` (a moment reset some training recipes do) must not leave the cached launch plan
+    stepping the discarded state tensors: the next step starts from fresh zero moments, like a new optimizer."""
+    fo = _fo()
+    shapes = [5000, 4096, 70001]
+    pa = _make_params(shapes, torch.bfloat16, 70)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")   # pure bf16 training is remarked on
+        oa = fo.FlashAdamW(pa, lr=1e-3, master_weight_bits=None, quantize=True)
+    for it in range(3):
+        _set_grads(pa, 700 + it)
+        oa.step()
+    oa.state.clear()
+    pb = [nn.Parameter(p.detach().clone()) for p in pa]
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        ob = fo.FlashAdamW(pb, lr=1e-3, master_weight_bits=None, quantize=True)
+    for it in range(2):
+        _set_grads(pa, 710 + it)
+        _set_grads(pb, 710 + it)
+        oa.step()
+        ob.step()
+    for a, b in zip(pa, pb):
+        assert torch.equal(a, b)
+        sa, sb = _state_tensors(oa, a), _state_tensors(ob, b)
+        for k in sa:
+            assert parity.bits_equal(sa[k], sb[k]), k
+        assert float(oa.state[a]["step"]) == 2.0
