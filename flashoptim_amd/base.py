@@ -459,6 +459,14 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
                 return False
         moved = []
         for b in cache.buckets:
+            if b.step_pool is not None:
+                # the counters are live state the caller may have rewritten (a warm restart zeroes them): take the
+                # step number from them, and leave counters that no longer agree to the per-parameter path
+                lo, hi = torch.aminmax(b.step_pool)
+                lo = lo.item()
+                if lo != hi.item():
+                    return False
+                b.step_value = int(lo)
             if b.plan is None:  # single-tensor bucket: launched from the live tensors below
                 for p in b.params:
                     g = p.grad

@@ -1128,3 +1128,31 @@ def test_clearing_the_optimizer_state_restarts_the_moments():
         for k in sa:
             assert parity.bits_equal(sa[k], sb[k]), k
         assert float(oa.state[a]["step"]) == 2.0
+
+
+def test_rewritten_step_counters_are_honoured_by_the_cached_plan():
+    """The per-parameter `step` scalars are ordinary state: zeroing them (a warm restart of the bias correction)
+    or setting one of them apart must steer the next cached step exactly as it steers per-tensor stepping."""
+    fo = _fo()
+    shapes = [5000, 4096, 70001]
+    pa, pb = _make_params(shapes, torch.bfloat16, 80), _make_params(shapes, torch.bfloat16, 80)
+    oa, ob = fo.FlashAdamW(pa, lr=1e-3), fo.FlashAdamW(pb, lr=1e-3)
+    for it in range(8):
+        _set_grads(pa, 800 + it)
+        _set_grads(pb, 800 + it)
+        if it == 3:      # warm restart: every counter back to zero
+            for opt in (oa, ob):
+                for st in opt.state.values():
+                    st["step"].zero_()
+        if it == 5:      # one parameter set apart
+            oa.state[pa[1]]["step"].fill_(40.0)
+            ob.state[pb[1]]["step"].fill_(40.0)
+        oa.step()
+        for p in pb:
+            ob.step_param(p)
+    for a, b in zip(pa, pb):
+        assert torch.equal(a, b)
+        sa, sb = _state_tensors(oa, a), _state_tensors(ob, b)
+        for k in sa:
+            assert parity.bits_equal(sa[k], sb[k]), k
+    assert [float(oa.state[p]["step"]) for p in pa] == [5.0, 43.0, 5.0]
