@@ -57,6 +57,7 @@ class LaunchKey:
     ecc_bytes: int
     quantized: bool
     scalars: tuple            # keyword arguments of the kernel wrapper, as a sorted tuple of items
+    device: Optional[torch.device] = None   # one launch reaches one device's memory only
 
 
 @dataclass
@@ -327,7 +328,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         mom = param_state[mom_name] if mom_name else None
         var = param_state[var_name] if var_name else None
         key = LaunchKey(kind, param.dtype, 0 if errors is None else errors.element_size(),
-                        mom.is_quantized() if mom is not None else False, tuple(sorted(scalars.items())))
+                        mom.is_quantized() if mom is not None else False, tuple(sorted(scalars.items())), param.device)
         tensors = StepTensors(
             param=param, grad=grad, ecc=errors,
             mom=None if mom is None else mom.kernel_tensor,
