@@ -305,6 +305,16 @@ def main() -> None:
     else:
         avg_device_ms = first.elapsed_time(last)
 
+    # a second pass with an event pair around every step, for the median and the fastest step (the pairs themselves
+    # cost a few microseconds per step, which is why the averages above come from the pass without them)
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for begin, end in pairs:
+        begin.record()
+        step()
+        end.record()
+    torch.cuda.synchronize()
+    per_step = sorted(begin.elapsed_time(end) for begin, end in pairs)
+
     step_bytes = work.get("copy_bytes", total * work["bpp"])
     achieved = step_bytes / (avg_device_ms * 1e-3) / 1e9
     out = {
@@ -329,6 +339,7 @@ def main() -> None:
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(args.workload),
             "step_device_ms_avg": avg_device_ms, "step_device_ms_avg_with_lead_in": first.elapsed_time(last) / args.steps,
+            "step_device_ms_median": per_step[len(per_step) // 2], "step_device_ms_min": per_step[0],
             "algorithmic_bytes_per_step": step_bytes,
         },
     }
