@@ -94,7 +94,13 @@ def lib() -> ctypes.CDLL:
                     )
                 handle = ctypes.CDLL(_LIB_PATH)
                 for name, (restype, argtypes) in SIGNATURES.items():
-                    fn = getattr(handle, name)
+                    try:
+                        fn = getattr(handle, name)
+                    except AttributeError:
+                        raise RuntimeError(
+                            f"{_LIB_PATH} does not export {name}: it was built from older sources. Rebuild it with "
+                            "`make -C flashoptim_amd/csrc`."
+                        ) from None
                     fn.restype = restype
                     fn.argtypes = argtypes
                 _lib = handle
