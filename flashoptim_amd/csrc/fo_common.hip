@@ -48,23 +48,12 @@ int check_hip(hipError_t e, const char* what) {
 
 const char* last_error() { return g_err; }
 
-static int env_int(const char* name, int fallback) {
-    const char* e = getenv(name);
-    const int v = e ? atoi(e) : 0;
-    return (v >= 1 && v <= 1024) ? v : fallback;
-}
-
-int step_lds_pad_bytes() {
+int debug_workgroups_per_cu() {
     static const int value = [] {
-        const char* e = getenv("FO_STEP_LDS_PAD");
-        const int v = e ? atoi(e) : -1;
-        return (v >= 0 && v <= 64 * 1024) ? v : -1;
+        const char* e = getenv("FO_DEBUG_WG_PER_CU");
+        const int v = e ? atoi(e) : 0;
+        return (v >= 1 && v <= 32) ? v : 0;
     }();
-    return value;
-}
-
-int default_tiles_per_chunk() {
-    static const int value = env_int("FO_TILES_PER_CHUNK", 1);
     return value;
 }
 
@@ -105,7 +94,7 @@ int fo_device_compute_units(int device) {
 
 int64_t fo_count_chunks(const int64_t* numels, int64_t n_tensors, int tiles_per_chunk) {
     if (!numels || n_tensors < 0) return fail(FO_ERR_INVALID_ARGUMENT, "bad tensor length array");
-    const int64_t tpc = tiles_per_chunk > 0 ? tiles_per_chunk : default_tiles_per_chunk();
+    const int64_t tpc = tiles_per_chunk > 0 ? tiles_per_chunk : 1;
     int64_t total = 0;
     for (int64_t i = 0; i < n_tensors; ++i) {
         if (numels[i] < 0) return fail(FO_ERR_INVALID_ARGUMENT, "tensor %lld has negative length", (long long)i);
@@ -120,7 +109,7 @@ int64_t fo_build_chunks(const int64_t* numels, int64_t n_tensors, int tiles_per_
     if (need < 0) return need;
     if (!out || capacity < need) return fail(FO_ERR_INVALID_ARGUMENT, "chunk buffer too small (%lld < %lld)", (long long)capacity, (long long)need);
     if (n_tensors > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "too many tensors");
-    const int64_t tpc = tiles_per_chunk > 0 ? tiles_per_chunk : default_tiles_per_chunk();
+    const int64_t tpc = tiles_per_chunk > 0 ? tiles_per_chunk : 1;
     int64_t c = 0;
     for (int64_t i = 0; i < n_tensors; ++i) {
         const int64_t tiles = (numels[i] + fo::kTileElems - 1) / fo::kTileElems;

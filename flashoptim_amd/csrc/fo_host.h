@@ -15,13 +15,9 @@ int check_hip(hipError_t e, const char* what);
 int compute_units();
 const char* last_error();
 
-// Override, from FO_STEP_LDS_PAD in the environment, of the unused dynamic LDS that every step-kernel workgroup
-// requests to bound the workgroups resident on a compute unit; -1 when unset (read once; for tuning).
-int step_lds_pad_bytes();
-
-// Tiles per work item of the multi-tensor chunk table when the caller passes tiles_per_chunk <= 0.
-// FO_TILES_PER_CHUNK in the environment overrides it (read once; for tuning).
-int default_tiles_per_chunk();
+// The library's one debug switch: FO_DEBUG_WG_PER_CU=<n> in the environment (read once) makes every step kernel
+// cap its residency at n workgroups per compute unit instead of its own measured optimum; 0 when unset.
+int debug_workgroups_per_cu();
 
 // Shared argument check of the multi-tensor entry points: counts, dtype code and table pointers.
 int validate_multi_tables(const void* descs, int64_t n_tensors, const void* chunks, int64_t n_chunks, int dtype);

@@ -1,0 +1,358 @@
+// Per-element arithmetic of the gfx950 step kernels, in one place and in a form that also compiles for the
+// host: the ECC join/split, the moment requantiser and the Adam / SGD / Lion element updates.  The kernels
+// (fo_adam.hip, fo_momentum.hip, fo_codec.hip) call exactly these functions; a CPU build of the same text
+// (FO_MATH_HOST defined, any C++17 compiler) lets the arithmetic be compared element for element with an IEEE
+// evaluation of the reference formulas on a machine without a GPU.
+//
+// Nothing here touches memory, lanes or LDS.  fp32 throughout; the translation units are compiled with
+// -ffp-contract=off, so a fused multiply-add happens only where fmaf() is written.
+//
+// The kernels lean on four hardware approximations (v_rcp_f32, v_rsq_f32, v_sqrt_f32: within one ulp, correctly
+// rounded for 85-90 % of inputs on MI355X) and on a few exact instructions (v_ldexp_f32, v_med3, v_cvt_flr).
+// In the host build they are stand-ins with the same contract; `fo_math_host_noise` != 0 makes the approximate
+// ones err by an ulp in a pseudo-random direction, which is how the CPU tests show that every result that
+// is meant to be correctly rounded stays so whatever the hardware returns inside its error bound.
+//
+// "ref:" cites /root/reference/flashoptim/optimizers.py.
+#pragma once
+
+#include <stdint.h>
+
+#include <cmath>
+#include <limits>
+
+#ifdef FO_MATH_HOST
+#include <math.h>
+#define FO_FN static inline
+#else
+#include <hip/hip_runtime.h>
+#define FO_FN __device__ __forceinline__
+#endif
+
+namespace fo {
+
+typedef uint32_t u32;
+
+constexpr int kGroup = 32;             // ref:1549, 2219: quantisation group
+constexpr float kMagic = 12582912.0f;  // 1.5 * 2^23: x + kMagic leaves rne(x) in the low mantissa bits
+
+enum { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2 };
+
+template <int DT> struct DTypeInfo;
+template <> struct DTypeInfo<DT_F32> { static constexpr int bytes = 4, mant = 23, epl = 4; };
+template <> struct DTypeInfo<DT_BF16> { static constexpr int bytes = 2, mant = 7, epl = 8; };
+template <> struct DTypeInfo<DT_F16> { static constexpr int bytes = 2, mant = 10, epl = 8; };
+
+FO_FN float as_f32(u32 u) { return __builtin_bit_cast(float, u); }
+FO_FN u32 as_u32(float f) { return __builtin_bit_cast(u32, f); }
+
+// ------------------------------------------------------------------------------------------------
+// the instructions the kernels rely on
+// ------------------------------------------------------------------------------------------------
+namespace hw {
+#ifdef FO_MATH_HOST
+extern "C" int fo_math_host_noise;
+// Moves an approximate result one ulp up or down for about a quarter of the inputs each.
+static inline float nudge(float exact, float x) {
+    if (!fo_math_host_noise || !(exact == exact) || exact == 0.0f || __builtin_isinf(exact)) return exact;
+    u32 h = as_u32(x) * 2654435761u + (u32)fo_math_host_noise * 40503u;
+    h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+    const u32 pick = h & 3u;
+    if (pick == 0) return as_f32(as_u32(exact) + 1u);
+    if (pick == 1) return as_f32(as_u32(exact) - 1u);
+    return exact;
+}
+static inline float rcp(float x) { return nudge((float)(1.0 / (double)x), x); }
+static inline float rsq(float x) { return nudge((float)(1.0 / sqrt((double)x)), x); }
+static inline float ldexp(float x, int e) { return ldexpf(x, e); }
+static inline float med3(float x, float lo, float hi) { return fminf(fmaxf(x, lo), hi); }
+static inline int floor_to_int(float x) { return (int)floorf(x); }
+static inline float fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+#else
+FO_FN float rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+FO_FN float rsq(float x) { return __builtin_amdgcn_rsqf(x); }
+FO_FN float ldexp(float x, int e) { return __builtin_amdgcn_ldexpf(x, e); }
+FO_FN float med3(float x, float lo, float hi) { return __builtin_amdgcn_fmed3f(x, lo, hi); }
+// (int)floor(x) in one instruction
+FO_FN int floor_to_int(float x) {
+    int r;
+    asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(r) : "v"(x));
+    return r;
+}
+FO_FN float fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+#endif
+FO_FN u32 clamp_u32(u32 x, u32 lo, u32 hi) {  // one v_med3_u32
+    const u32 t = x > lo ? x : lo;
+    return t < hi ? t : hi;
+}
+}  // namespace hw
+
+// ------------------------------------------------------------------------------------------------
+// correctly rounded quotients and roots from the approximate instructions
+// ------------------------------------------------------------------------------------------------
+
+// RN(a / b) given r within an ulp of 1/b: one residual correction of the quotient estimate.  q + rem * r equals
+// a/b to about 2^-22 ulp before the final rounding of the fma, so the result is the correctly rounded quotient
+// except when a/b lies that close to a rounding boundary (about one quotient in a million); with r = RN(1/b)
+// it is correctly rounded always (Markstein).  No scaling: callers keep b well inside the normal range.
+FO_FN float div_corrected(float a, float b, float r) {
+    const float q = a * r;
+    const float rem = hw::fma(-b, q, a);
+    return hw::fma(rem, r, q);
+}
+
+// RN(sqrt(x)) for x >= 0 from the reciprocal-root instruction: s = x * y, one Newton correction with the exact
+// residual x - s*s.  x == 0 gives 0 (the clamp keeps y finite), subnormal x gives a value below 2^-63.
+FO_FN float sqrt_corrected(float x) {
+    const float y = hw::rsq(fmaxf(x, 1.17549435e-38f));
+    const float s = x * y;
+    const float h = 0.5f * y;
+    const float rem = hw::fma(-s, s, x);
+    return hw::fma(rem, h, s);
+}
+
+// ------------------------------------------------------------------------------------------------
+// ECC: narrow value + signed integer fraction of half its ulp (ref:2682-2776)
+// ------------------------------------------------------------------------------------------------
+template <int ECCB> struct EccInfo;
+template <> struct EccInfo<1> { static constexpr float max_val = 127.0f; };      // ref:1521
+template <> struct EccInfo<2> { static constexpr float max_val = 32767.0f; };    // ref:1523
+
+// fp32 bit pattern of 2^E, E = unbiased exponent of the narrow value with zero/subnormal mapped to the
+// smallest normal exponent (ref:2704-2712), given the value widened to fp32.  bf16 shares fp32's exponent
+// field; an fp16 subnormal widens to an fp32 normal below 2^-14, which the lower clamp maps back to -14.
+// The upper clamp keeps inf/NaN inputs from producing an infinite scale.
+template <int DT> FO_FN u32 pow2_of_exponent_bits(float widened) {
+    constexpr u32 lo = (DT == DT_F16) ? ((127u - 14u) << 23) : (1u << 23);
+    const u32 e = as_u32(widened) & 0x7f800000u;
+    return hw::clamp_u32(e, lo, 254u << 23);
+}
+
+// x_narrow + (ecc / MAX) * 2^(E - mant - 1) with the product and the sum fused (ref:2767-2776; the reference
+// compiles with FP fusion, and its invariants test only passes with the fused form).
+//   ecc_fraction: (ecc / MAX) * 2^-(mant+1), the division correctly rounded, formed as fma(e, K_hi, e * K_lo) with
+//   K_hi + K_lo = 2^-(mant+1) / MAX to well beyond fp32 precision (checked exhaustively over every int8 / int16
+//   value on the host).  For int8 codes the kernels read the same values from a 256-entry table (EccFractionTable).
+template <int DT, int ECCB> FO_FN float ecc_fraction(float ecc) {
+    constexpr double k = 1.0 / ((double)EccInfo<ECCB>::max_val * (double)(1 << (DTypeInfo<DT>::mant + 1)));
+    constexpr float k_hi = (float)k;
+    constexpr float k_lo = (float)(k - (double)k_hi);
+    return hw::fma(ecc, k_hi, ecc * k_lo);
+}
+template <int DT> FO_FN float ecc_join_fraction(float widened, float fraction) {
+    return hw::fma(fraction, as_f32(pow2_of_exponent_bits<DT>(widened)), widened);
+}
+template <int DT, int ECCB> FO_FN float ecc_join(float widened, float ecc) {
+    return ecc_join_fraction<DT>(widened, ecc_fraction<DT, ECCB>(ecc));
+}
+
+// Signed fraction of half an ulp of the NEW narrow value, scaled to +-MAX and rounded half away from zero
+// (ref:2735-2756).  Returns a word whose low byte / half is the two's-complement code.
+//   General form: sc = clamp(en) * MAX rounded to fp32 as in the reference, then trunc(sc + copysign(0.5, sc)),
+//   which equals copysign(floor(|sc| + 0.5), sc) including the fp32 rounding of the sum.
+//   bf16 with an int8 code: p - narrow is exact and a multiple of 2^-16 half-ulps, so en * 127 fits 24 bits and
+//   is exact; the only tie that can occur is +-63.5, where half-even and half-away agree.  One fma against
+//   1.5 * 2^23 then leaves the rounded integer in the low mantissa bits.
+//   CLAMP = false is for callers whose narrow value IS the round-to-nearest of p (|en| <= 1 by construction).
+//   For them the bf16/int8 case folds the scaling into the fma: with eb the biased exponent field of the narrow
+//   value (1..254), en * 127 = err * 127 * 2^(135 - eb).  That factor can exceed the fp32 range, so both fma
+//   operands carry an extra 2^-13: S = 127 * 2^(122 - eb) is a normal number for every eb (bit pattern
+//   0x7ffe0000 - (eb << 23)) and 1.5 * 2^10 + en * 127 * 2^-13 has the same mantissa bits as
+//   1.5 * 2^23 + en * 127, rounded at the same place.
+template <int DT, int ECCB, bool CLAMP> FO_FN u32 ecc_split_bits(float p, float widened) {
+    const float err = p - widened;
+    if constexpr (DT == DT_BF16 && ECCB == 1 && !CLAMP) {
+        const float s = as_f32(0x7ffe0000u - pow2_of_exponent_bits<DT>(widened));
+        return as_u32(hw::fma(err, s, 1536.0f));
+    } else {
+        const int nls = (DTypeInfo<DT>::mant + 1 + 127) - (int)(pow2_of_exponent_bits<DT>(widened) >> 23);
+        float en = hw::ldexp(err, nls);
+        if constexpr (CLAMP) en = hw::med3(en, -1.0f, 1.0f);
+        if constexpr (DT == DT_BF16 && ECCB == 1) {
+            return as_u32(hw::fma(en, EccInfo<ECCB>::max_val, kMagic));
+        } else {
+            const float sc = en * EccInfo<ECCB>::max_val;
+            return (u32)(int)(sc + __builtin_copysignf(0.5f, sc));
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// 8-bit group codec
+// ------------------------------------------------------------------------------------------------
+
+// The two code tables of the step kernels, evaluated by the compiler (IEEE, round to nearest):
+//   v[b]        first-moment value of signed code byte b before the group scale, (q/127) / (2 - |q/127|) with
+//               each operation correctly rounded (ref:2332-2336);
+//   v[256 + b]  (q/127) * 2^-(mant+1) for an int8 ECC byte b, the division correctly rounded (ref:2772): the
+//               factor that multiplies 2^E in ecc_join_fraction.  The scaling by a power of two is exact.
+template <int DT> struct StepTables {
+    float v[512];
+    constexpr StepTables() : v() {
+        for (int b = 0; b < 256; ++b) {
+            const int q = b < 128 ? b : b - 256;
+            const float y = (float)q / 127.0f;
+            const float a = y < 0.0f ? -y : y;
+            v[b] = y / (2.0f - a);
+            v[256 + b] = y * (1.0f / (float)(1 << (DTypeInfo<DT>::mant + 1)));
+        }
+    }
+};
+typedef StepTables<DT_BF16> SoftsignTable;  // first 256 entries: the same for every parameter dtype
+
+// Requantisation of a moment value against its group's absmax, rounding exactly as the reference's formula does
+// when every operation is evaluated in IEEE fp32 (ref:2405-2419, 1703-1710):
+//     nm = m / am;  t = (2 nm) / (1 + |nm|);  code = floor(t * 127 + 0.5)          first moment
+//     code = floor((r / av) * 255 + 0.5),  r = sqrt(v)                             second moment
+// Each quotient is the correctly rounded one (div_corrected), the product and the sum round separately, and the
+// floor is taken of the rounded sum.  Doubling is exact, so RN(2nm / d) * 127 is formed as RN(nm / d) * 254.
+// ram / rav: the reciprocal instruction applied to the group absmax (shared by the lanes of the group).
+// Returns a word whose low byte is the code.
+FO_FN u32 quantize_mom_code(float m, float am, float ram) {
+    const float nm = div_corrected(m, am, ram);
+    const float d = 1.0f + fabsf(nm);
+    const float t = div_corrected(nm, d, hw::rcp(d));
+    return (u32)hw::floor_to_int(t * 254.0f + 0.5f);
+}
+FO_FN u32 quantize_var_code(float r, float av, float rav) {
+    const float q = div_corrected(r, av, rav);
+    return (u32)(int)(q * 255.0f + 0.5f);  // non-negative: truncation is the floor
+}
+
+// ------------------------------------------------------------------------------------------------
+// Adam / AdamW element update (ref:2296-2375)
+// ------------------------------------------------------------------------------------------------
+
+// Per-launch constants.  Scalars arrive as fp32 like the reference's kernel arguments; 1 - x is formed in fp32
+// (ref:2357-2364).
+struct AdamHyper {
+    float b1, one_m_b1, b2, one_m_b2, wd, one_m_wd;
+    // folded form: the per-step bias corrections and the learning rate are folded on the host (in double, rounded
+    // once) into the two constants of the update's denominator, negated so that the update is one fma:
+    //     lr * (m / bc1) / (sqrt(v / bc2) + eps)  ==  m / (sqrt(v) * den_scale + den_bias)
+    //     den_scale = bc1 / (lr * sqrt(bc2)),  den_bias = eps * bc1 / lr
+    float neg_den_scale, neg_den_bias;
+    float sqrt_b2_over_255;  // dequantised sqrt(v_old * b2) = code * scale * sqrt(b2) / 255
+    // operation-by-operation form (EXACT): the reference's own sequence with correctly rounded quotients
+    float lr, eps, bc1, rcp_bc1, bc2, rcp_bc2;  // rcp_*: correctly rounded reciprocals, formed on the host
+};
+
+// Host side: the constants of one launch from the reference's kernel arguments (ref:2264-2270).
+inline AdamHyper make_adam_hyper(float lr, float beta1, float beta2, float eps, float wd, int step) {
+    AdamHyper h;
+    h.b1 = beta1; h.one_m_b1 = 1.0f - beta1;
+    h.b2 = beta2; h.one_m_b2 = 1.0f - beta2;
+    h.wd = wd; h.one_m_wd = 1.0f - wd;
+    h.sqrt_b2_over_255 = (float)(std::sqrt((double)beta2) / 255.0);
+    // beta^step is the correctly rounded fp32 power, 1 - that is formed in fp32 (ref:2368-2369)
+    h.bc1 = 1.0f - (float)std::pow((double)beta1, (double)step);
+    h.bc2 = 1.0f - (float)std::pow((double)beta2, (double)step);
+    h.rcp_bc1 = (float)(1.0 / (double)h.bc1);
+    h.rcp_bc2 = (float)(1.0 / (double)h.bc2);
+    h.lr = lr; h.eps = eps;
+    const double bc1 = (double)h.bc1, bc2 = (double)h.bc2;
+    if (lr != 0.0f) {
+        h.neg_den_scale = -(float)(bc1 / ((double)lr * std::sqrt(bc2)));
+        h.neg_den_bias = -(float)((double)eps * bc1 / (double)lr);
+    } else {  // no update: the denominator is infinite whatever sqrt(v) is
+        h.neg_den_scale = 0.0f;
+        h.neg_den_bias = -std::numeric_limits<float>::infinity();
+    }
+    return h;
+}
+
+// Which variants follow the reference's update operation by operation (EXACT) instead of the folded form:
+// fp32 parameters, where one fp32 ulp is the master precision and the 16.25 bytes per element leave room
+// for the extra arithmetic.  Narrow parameters use the folded update (see adam_apply).
+#ifndef FO_EXACT_RULE
+#define FO_EXACT_RULE (DT == DT_F32)
+#endif
+template <int DT, int ECCB> struct AdamExact { static constexpr bool value = FO_EXACT_RULE; };
+
+// New moments from the dequantised pieces.
+//   EXACT = false: the EMA decay is folded into the group scale (one multiply per lane instead of one per
+//   element): m = fma(table[qm], sm * b1, g * (1 - b1)); v = fma(s, s, g^2 * (1 - b2)), s = qv * sv * sqrt(b2)/255.
+//   From an all-zero state both equal the reference's values bit for bit.
+//   EXACT = true: every operation of ref:2332-2360 rounded on its own.
+template <bool EXACT>
+FO_FN void adam_moments_quantized(float g, float table_m, float sm, float sm_b1, float qv, float sv, float sv_b2,
+                                  const AdamHyper& h, float& mn, float& vn) {
+    if constexpr (EXACT) {
+        const float mo = table_m * sm;                                              // ref:2332-2343
+        const float s = div_corrected(qv, 255.0f, 1.0f / 255.0f) * sv;               // ref:2333-2347
+        const float vo = s * s;                                                     // ref:2348
+        mn = mo * h.b1 + g * h.one_m_b1;                                            // ref:2357
+        vn = vo * h.b2 + (g * g) * h.one_m_b2;                                      // ref:2360
+    } else {
+        mn = hw::fma(table_m, sm_b1, g * h.one_m_b1);
+        const float s = qv * sv_b2;
+        vn = hw::fma(s, s, (g * g) * h.one_m_b2);
+    }
+}
+// Unquantised states: operation by operation as written in the reference, no contraction (ref:2351-2360).
+FO_FN void adam_moments_plain(float g, float mo, float vo, const AdamHyper& h, float& mn, float& vn) {
+    mn = mo * h.b1 + g * h.one_m_b1;
+    vn = vo * h.b2 + (g * g) * h.one_m_b2;
+}
+
+// p -= lr * (m/bc1) / (sqrt(v/bc2) + eps)  (ref:2368-2375).  r = sqrt(v), shared with the requantiser.
+template <bool EXACT> FO_FN float adam_apply(float p, float mn, float vn, float r, const AdamHyper& h) {
+    if constexpr (EXACT) {
+        const float cm = div_corrected(mn, h.bc1, h.rcp_bc1);
+        const float cv = div_corrected(vn, h.bc2, h.rcp_bc2);
+        const float den = sqrt_corrected(cv) + h.eps;
+        float rd = hw::rcp(den);
+        rd = hw::fma(hw::fma(-den, rd, 1.0f), rd, rd);  // reciprocal refined to well below an ulp
+        return p - div_corrected(h.lr * cm, den, rd);
+    } else {
+        const float neg_den = hw::fma(r, h.neg_den_scale, h.neg_den_bias);
+        return hw::fma(mn, hw::rcp(neg_den), p);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// SGD / SGDW / Nesterov / Lion element update (ref:1624-1683, 1447-1465)
+// ------------------------------------------------------------------------------------------------
+enum { KIND_SGD = 0, KIND_LION = 1, KIND_PLAIN = 2 };
+
+struct MomentumHyper {
+    float lr, mom_coef, update_coef, one_m_mom_coef, one_m_update_coef, wd, one_m_wd;
+    int decoupled, nesterov;
+    int apply_decay;  // momentum-free branch only: the reference skips both decays when weight_decay == 0
+};
+
+inline MomentumHyper make_momentum_hyper(float lr, float mom_coef, float update_coef, float wd, int decoupled, int nesterov) {
+    MomentumHyper h;
+    h.lr = lr; h.mom_coef = mom_coef; h.update_coef = update_coef;
+    h.one_m_mom_coef = 1.0f - mom_coef; h.one_m_update_coef = 1.0f - update_coef;
+    h.wd = wd; h.one_m_wd = 1.0f - wd;
+    h.decoupled = decoupled ? 1 : 0; h.nesterov = nesterov ? 1 : 0;
+    h.apply_decay = wd > 0.0f ? 1 : 0;
+    return h;
+}
+
+// g, p: gradient and master weight; mo: the dequantised (or plain) momentum.  Writes the new weight and momentum.
+template <int KIND> FO_FN void momentum_element(float g, float& p, float mo, const MomentumHyper& h, float& mn) {
+    float pk = p;
+    if constexpr (KIND == KIND_PLAIN) {
+        if (h.apply_decay && !h.decoupled) g = g + pk * h.wd;                       // ref:1452-1453
+        if (h.apply_decay && h.decoupled) pk = pk * h.one_m_wd;                     // ref:1454-1455
+        pk = pk - g * h.lr;                                                         // ref:1456
+        mn = 0.0f;
+    } else if constexpr (KIND == KIND_LION) {
+        const float u = (mo * h.update_coef) + (g * h.one_m_update_coef);           // ref:1667
+        const float sgn = (u > 0.0f) ? 1.0f : ((u < 0.0f) ? -1.0f : 0.0f);          // ref:1668
+        mn = (mo * h.mom_coef) + (g * h.one_m_mom_coef);                            // ref:1669
+        pk = pk * h.one_m_wd;                                                       // ref:1675
+        pk = pk - sgn * h.lr;                                                       // ref:1676
+    } else {
+        if (!h.decoupled) g = g + pk * h.wd;                                        // ref:1639-1640
+        mn = mo * h.mom_coef + g * h.update_coef;                                   // ref:1671
+        if (h.decoupled) pk = pk * h.one_m_wd;                                      // ref:1678-1679
+        if (h.nesterov) pk = pk - (g + h.mom_coef * mn) * h.lr;                     // ref:1680-1681
+        else pk = pk - mn * h.lr;                                                   // ref:1682-1683
+    }
+    p = pk;
+}
+
+}  // namespace fo

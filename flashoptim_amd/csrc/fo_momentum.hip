@@ -7,14 +7,6 @@ namespace fo {
 // ------------------------------------------------------------------------------------------------
 // SGD / SGDW / Nesterov / Lion / momentum-free SGD (ref:1586-1719, 1447-1465)
 // ------------------------------------------------------------------------------------------------
-enum { KIND_SGD = 0, KIND_LION = 1, KIND_PLAIN = 2 };
-
-struct MomentumHyper {
-    float lr, mom_coef, update_coef, one_m_mom_coef, one_m_update_coef, wd, one_m_wd;
-    int decoupled, nesterov;
-    int apply_decay;  // momentum-free branch only: the reference skips both decays when weight_decay == 0
-};
-
 template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumRaw {
     static constexpr int EPL = DTypeInfo<DT>::epl;
     static constexpr int SB = (KIND == KIND_PLAIN) ? 0 : (QUANT ? 1 : DTypeInfo<DT>::bytes);
@@ -25,67 +17,46 @@ template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumRaw {
 };
 
 template <int DT, int ECCB, bool QUANT, int KIND, int FAST>
-__device__ __forceinline__ void momentum_load(const TensorPtrs& t, int64_t first, MomentumRaw<DT, ECCB, QUANT, KIND>& r) {
+__device__ __forceinline__ void momentum_load(const TensorPtrs& t, Where w, MomentumRaw<DT, ECCB, QUANT, KIND>& r) {
     constexpr int EPL = DTypeInfo<DT>::epl;
     constexpr int PB = DTypeInfo<DT>::bytes;
     constexpr int SB = MomentumRaw<DT, ECCB, QUANT, KIND>::SB;
     const int64_t n = t.n;
-    load_lane<PB, EPL, FAST>(r.g, t.grad, first, n);
-    load_lane<PB, EPL, FAST>(r.p, t.param, first, n);
-    load_lane<ECCB, EPL, FAST>(r.e, t.ecc, first, n);
-    load_lane<SB, EPL, FAST>(r.m, t.mom, first, n);
+    load_lane<PB, EPL, FAST>(r.g, t.grad, w, n);
+    load_lane<PB, EPL, FAST>(r.p, t.param, w, n);
+    load_lane<ECCB, EPL, FAST>(r.e, t.ecc, w, n);
+    load_lane<SB, EPL, FAST>(r.m, t.mom, w, n);
     r.sm = 0x3c00;  // 1.0
     if constexpr (QUANT && KIND != KIND_PLAIN) {
-        if (FAST == kVector || first < n) r.sm = t.mom_scales[first >> 5];                     // ref:1645-1646
+        if (FAST == kVector || w.first() < n) r.sm = load_scale(t.mom_scales, w);                     // ref:1645-1646
     }
 }
 
 template <int DT, int ECCB, bool QUANT, int KIND, int FAST>
-__device__ __forceinline__ void momentum_finish(const TensorPtrs& t, int64_t first, MomentumRaw<DT, ECCB, QUANT, KIND>& raw,
-                                                const MomentumHyper& h, const float* lut_lane) {
+__device__ __forceinline__ void momentum_finish(const TensorPtrs& t, Where w, MomentumRaw<DT, ECCB, QUANT, KIND>& raw,
+                                                const MomentumHyper& h, const float* lut) {
     constexpr int EPL = DTypeInfo<DT>::epl;
     constexpr int PB = DTypeInfo<DT>::bytes;
     constexpr int SB = MomentumRaw<DT, ECCB, QUANT, KIND>::SB;
     const int64_t n = t.n;
-    const bool live_group = FAST == kVector || first < n;
-    const int64_t group = first >> 5;
+    const bool live_group = FAST == kVector || w.first() < n;
     const float sm = f16_bits_to_f32(raw.sm);
 
     float p[EPL], m[EPL];
-    read_master<DT, ECCB, EPL>(p, raw.p, raw.e);
+    read_master<DT, ECCB, EPL>(p, raw.p, raw.e, lut);
 
-    float am = 0.0f;
 #pragma unroll
     for (int k = 0; k < EPL; ++k) {
-        float g = widen<DT, EPL>(raw.g, k);
-        float pk = p[k];
-        if constexpr (KIND == KIND_PLAIN) {
-            if (h.apply_decay && !h.decoupled) g = g + pk * h.wd;                   // ref:1452-1453
-            if (h.apply_decay && h.decoupled) pk = pk * h.one_m_wd;                 // ref:1454-1455
-            pk = pk - g * h.lr;                                                     // ref:1456
-        } else {
-            if (KIND == KIND_SGD && !h.decoupled) g = g + pk * h.wd;                // ref:1639-1640
-            float mo;
-            if constexpr (QUANT) mo = StepLut::lookup(lut_lane, byte_of<EPL>(raw.m, k)) * sm;   // ref:1648-1657
-            else mo = widen<DT, EPL>(raw.m, k);                                     // ref:1660-1661
-            float mn;
-            if constexpr (KIND == KIND_LION) {
-                const float u = (mo * h.update_coef) + (g * h.one_m_update_coef);        // ref:1667
-                const float sgn = (u > 0.0f) ? 1.0f : ((u < 0.0f) ? -1.0f : 0.0f);      // ref:1668
-                mn = (mo * h.mom_coef) + (g * h.one_m_mom_coef);                         // ref:1669
-                pk = pk * h.one_m_wd;                                                    // ref:1675
-                pk = pk - sgn * h.lr;                                                    // ref:1676
-            } else {
-                mn = mo * h.mom_coef + g * h.update_coef;                                // ref:1671
-                if (h.decoupled) pk = pk * h.one_m_wd;                                   // ref:1678-1679
-                if (h.nesterov) pk = pk - (g + h.mom_coef * mn) * h.lr;                  // ref:1680-1681
-                else pk = pk - mn * h.lr;                                                // ref:1682-1683
-            }
-            m[k] = mn;
+        const float g = widen<DT, EPL>(raw.g, k);
+        float mo = 0.0f;
+        if constexpr (KIND != KIND_PLAIN) {
+            if constexpr (QUANT) mo = lookup_mom(lut, byte_of<EPL>(raw.m, k)) * sm;        // ref:1648-1657
+            else mo = widen<DT, EPL>(raw.m, k);                                                 // ref:1660-1661
         }
-        p[k] = pk;
+        momentum_element<KIND>(g, p[k], mo, h, m[k]);
     }
 
+    float am = 0.0f;
     if constexpr (KIND != KIND_PLAIN) {
 #pragma unroll
         for (int k = 0; k < EPL; k += 2) am = fmaxf(fmaxf(am, fabsf(m[k])), fabsf(m[k + 1]));
@@ -93,34 +64,35 @@ __device__ __forceinline__ void momentum_finish(const TensorPtrs& t, int64_t fir
 
     Pack<ECCB, EPL> eout;
     write_master<DT, ECCB, EPL>(p, raw.p, eout);                                    // ref:1684-1694
-    store_lane<PB, EPL, FAST>(raw.p, t.param, first, n);
-    store_lane<ECCB, EPL, FAST>(eout, t.ecc, first, n);
+    store_lane<PB, EPL, FAST>(raw.p, t.param, w, n);
+    store_lane<ECCB, EPL, FAST>(eout, t.ecc, w, n);
 
     if constexpr (KIND != KIND_PLAIN) {
         if constexpr (QUANT) {
             am = fmaxf(group_max<EPL>(am), 1e-12f);                                 // ref:1702-1703
             quantize_mom<EPL>(m, am, raw.m);
-            store_lane<1, EPL, FAST>(raw.m, t.mom, first, n);
-            if (live_group && (threadIdx.x & (32 / EPL - 1)) == 0) store_scale(t.mom_scales, group, f32_to_f16_bits(am));  // ref:1713-1716
+            store_lane<1, EPL, FAST>(raw.m, t.mom, w, n);
+            if (live_group && (threadIdx.x & (32 / EPL - 1)) == 0) store_scale(t.mom_scales, w, f32_to_f16_bits(am));  // ref:1713-1716
         } else {
             narrow_all<DT, EPL>(m, raw.m);                                          // ref:1717-1719
-            store_lane<SB, EPL, FAST>(raw.m, t.mom, first, n);
+            store_lane<SB, EPL, FAST>(raw.m, t.mom, w, n);
         }
     }
 }
 
 template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumOp {
     using Hyper = MomentumHyper;
-    static constexpr bool kNeedsLut = QUANT && KIND != KIND_PLAIN;
-    static constexpr int kLdsBytes = 7936;  // 20 resident workgroups: measured optimum on MI355X (3 KiB of loads per wavefront)
+    static constexpr int kLutTables = ECCB == 1 ? 2 : ((QUANT && KIND != KIND_PLAIN) ? 1 : 0);  // LDS code tables (fo_device.h)
+    static constexpr int kDtype = DT;
+    static constexpr int kWorkgroupsPerCu = 24;  // measured on MI355X: 23 best for the 8B list, 26 for 4096 ragged tensors (3 KiB of loads per wavefront)
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = MomentumRaw<DT, ECCB, QUANT, KIND>;
-    template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, int64_t first, Raw& r) {
-        momentum_load<DT, ECCB, QUANT, KIND, FAST>(t, first, r);
+    template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {
+        momentum_load<DT, ECCB, QUANT, KIND, FAST>(t, w, r);
     }
     template <int FAST>
-    __device__ __forceinline__ static void finish(const TensorPtrs& t, int64_t first, Raw& r, const Hyper& h, const float* lut) {
-        momentum_finish<DT, ECCB, QUANT, KIND, FAST>(t, first, r, h, lut);
+    __device__ __forceinline__ static void finish(const TensorPtrs& t, Where w, Raw& r, const Hyper& h, const float* lut) {
+        momentum_finish<DT, ECCB, QUANT, KIND, FAST>(t, w, r, h, lut);
     }
 };
 
@@ -133,15 +105,7 @@ template <int DT, int EB, bool Q> using SgdOp = fo::MomentumOp<DT, EB, Q, fo::KI
 template <int DT, int EB, bool Q> using LionOp = fo::MomentumOp<DT, EB, Q, fo::KIND_LION>;
 template <int DT, int EB, bool Q> using PlainOp = fo::MomentumOp<DT, EB, Q, fo::KIND_PLAIN>;
 
-fo::MomentumHyper make_momentum_hyper(float lr, float mom_coef, float update_coef, float wd, int decoupled, int nesterov) {
-    fo::MomentumHyper h;
-    h.lr = lr; h.mom_coef = mom_coef; h.update_coef = update_coef;
-    h.one_m_mom_coef = 1.0f - mom_coef; h.one_m_update_coef = 1.0f - update_coef;
-    h.wd = wd; h.one_m_wd = 1.0f - wd;
-    h.decoupled = decoupled ? 1 : 0; h.nesterov = nesterov ? 1 : 0;
-    h.apply_decay = wd > 0.0f ? 1 : 0;
-    return h;
-}
+using fo::make_momentum_hyper;
 
 }  // namespace
 

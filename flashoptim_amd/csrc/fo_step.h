@@ -2,9 +2,8 @@
 // requantisation helpers, the two grid shapes (single tensor by value / chunk table over many tensors) and
 // the host-side launch + dispatch templates.
 //
-// Work decomposition.  A wavefront processes sub-tiles of 64 x EPL consecutive elements (EPL = 8 for bf16/fp16,
-// 4 for fp32; see fo_device.h for the access shape); a workgroup of FO_BLOCK_THREADS threads covers
-// FO_BLOCK_THREADS/64 x FO_SUBTILES_PER_WAVE neighbouring sub-tiles (its "span") and retires.  Workgroups are
+// Work decomposition.  A workgroup is one wavefront; it processes one "span" of 64 x EPL consecutive elements
+// (EPL = 8 for bf16/fp16, 4 for fp32; see fo_device.h for the access shape) and retires.  Workgroups are
 // deliberately tiny and short-lived: streaming from HBM is measurably better with many one-wavefront workgroups
 // that each touch every stream once than with larger or persistent ones.  The multi-tensor grid addresses work
 // through a chunk table in units of 4096-element tiles; a tile is an integer number of spans.  A quantisation
@@ -14,26 +13,15 @@
 // "ref:" cites /root/reference/flashoptim/optimizers.py.
 #pragma once
 
+#include <mutex>
+
 #include "fo_device.h"
 #include "fo_host.h"
 #include "../../include/flashoptim_hip.h"
 
-#ifndef FO_BLOCK_THREADS
-#define FO_BLOCK_THREADS 64
-#endif
-#ifndef FO_SUBTILES_PER_WAVE
-#define FO_SUBTILES_PER_WAVE 1
-#endif
-#ifndef FO_LUT_REPL
-#define FO_LUT_REPL 1
-#endif
-
 namespace fo {
 
-constexpr int kBlockThreads = FO_BLOCK_THREADS;
-constexpr int kBlockWaves = kBlockThreads / 64;
-constexpr int kPerWave = FO_SUBTILES_PER_WAVE;
-using StepLut = Lut<FO_LUT_REPL, kBlockThreads>;
+constexpr int kBlockThreads = 64;  // one wavefront per workgroup
 
 struct TensorPtrs {
     void* param;
@@ -65,13 +53,16 @@ __device__ __forceinline__ bool all_aligned16(const TensorPtrs& t) {
 // ------------------------------------------------------------------------------------------------
 
 // Reads the lane's parameter values as fp32 masters (ref:2299-2309).
+// An int8 ECC byte goes through the LDS table of correctly rounded fractions (one lookup instead of a convert and
+// two multiply-adds); int16 codes are converted arithmetically.
 template <int DT, int ECCB, int EPL>
 __device__ __forceinline__ void read_master(float (&p)[EPL], const Pack<DTypeInfo<DT>::bytes, EPL>& praw,
-                                            const Pack<ECCB, EPL>& eraw) {
+                                            const Pack<ECCB, EPL>& eraw, const float* lut) {
 #pragma unroll
     for (int k = 0; k < EPL; ++k) {
         const float w = widen<DT, EPL>(praw, k);
-        if constexpr (ECCB > 0) p[k] = ecc_join<DT, ECCB>(w, ecc_to_float<ECCB, EPL>(eraw, k));
+        if constexpr (ECCB == 1) p[k] = ecc_join_fraction<DT>(w, lookup_ecc(lut, byte_of<EPL>(eraw, k)));
+        else if constexpr (ECCB == 2) p[k] = ecc_join<DT, ECCB>(w, ecc_to_float<ECCB, EPL>(eraw, k));
         else p[k] = w;
     }
 }
@@ -93,28 +84,23 @@ __device__ __forceinline__ void write_master(const float (&p)[EPL], Pack<DTypeIn
     if constexpr (ECCB > 0) pack_codes<ECCB, EPL>(eb, eout);
 }
 
-// Quantises the lane's first-moment values against the group absmax `am` (shared by the group's lanes,
-// clamped at 1e-12): code = rne(127 * 2x/(1+|x|)), x = m/am  ==  rne(254 * m / (am + |m|))
-// (ref:2407-2418 with the two divisions merged algebraically; one hardware reciprocal per element).
+// Quantises the lane's first-moment values against the group absmax `am` (shared by the group's lanes, clamped
+// at 1e-12) and the lane's sqrt(v) values against the group maximum `av`; the rounding is the reference's
+// (fo_math.h: quantize_mom_code, quantize_var_code; ref:2405-2419, 1703-1710).
 template <int EPL>
 __device__ __forceinline__ void quantize_mom(const float (&m)[EPL], float am, Pack<1, EPL>& out) {
+    const float ram = hw::rcp(am);
     u32 b[EPL];
 #pragma unroll
-    for (int k = 0; k < EPL; ++k) {
-        const float t = m[k] * __builtin_amdgcn_rcpf(am + fabsf(m[k]));
-        b[k] = as_u32(fmaf(t, 254.0f, kMagic));
-    }
+    for (int k = 0; k < EPL; ++k) b[k] = quantize_mom_code(m[k], am, ram);
     pack_codes<1, EPL>(b, out);
 }
-
-// Quantises sqrt(v): code = rne(255 * r / av) with 255/av formed once per lane from the hardware reciprocal
-// (ref:2408-2419; av >= 1e-12, so the reciprocal is a normal number).
 template <int EPL>
 __device__ __forceinline__ void quantize_var(const float (&r)[EPL], float av, Pack<1, EPL>& out) {
-    const float scale = 255.0f * __builtin_amdgcn_rcpf(av);
+    const float rav = hw::rcp(av);
     u32 b[EPL];
 #pragma unroll
-    for (int k = 0; k < EPL; ++k) b[k] = as_u32(fmaf(r[k], scale, kMagic));
+    for (int k = 0; k < EPL; ++k) b[k] = quantize_var_code(r[k], av, rav);
     pack_codes<1, EPL>(b, out);
 }
 
@@ -131,12 +117,11 @@ __device__ __forceinline__ void narrow_all(const float (&x)[EPL], Pack<DTypeInfo
 // kernels
 // ------------------------------------------------------------------------------------------------
 
-// Elements one workgroup covers.
+// Elements one workgroup (= one wavefront) covers: 64 lanes x EPL.
 template <class Op> struct Span {
-    static constexpr int kSub = 64 * Op::kEpl;                       // elements per sub-tile
-    static constexpr int kElems = kBlockWaves * kPerWave * kSub;     // elements per workgroup
+    static constexpr int kElems = 64 * Op::kEpl;
     static constexpr int kPerTile = kTileElems / kElems;             // workgroups per 4096-element tile
-    static_assert(kElems <= kTileElems && kTileElems % kElems == 0, "a tile must be a whole number of workgroup spans");
+    static_assert(kTileElems % kElems == 0, "a tile must be a whole number of workgroup spans");
 };
 
 // Order of the spans.  The hardware deals workgroups round-robin to the 8 XCDs (workgroup b runs on XCD b % 8),
@@ -147,77 +132,65 @@ template <class Op> struct Span {
 // 1 KiB), so the identity order stays.
 
 // One span starting at element `base` of tensor t.  All loads are issued first, `between()` runs while they are
-// in flight (the workgroup commits the LDS table there), then the sub-tiles are finished one after the other.
+// in flight (the workgroup commits the LDS table there), then the span is finished.
 template <class Op, class Between>
 __device__ __forceinline__ void run_span(const TensorPtrs& t, int64_t base, bool aligned, const typename Op::Hyper& h,
-                                         const float* lut_lane, Between&& between) {
-    constexpr int kSub = Span<Op>::kSub;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    // wavefront w takes sub-tiles w, w + W, ... of the span
-    const int64_t first0 = base + (int64_t)wave * kSub + lane * Op::kEpl;
-    constexpr int64_t kStride = (int64_t)kBlockWaves * kSub;
-    typename Op::Raw raw[kPerWave];
+                                         const float* lut, Between&& between) {
+    const Where first{base, (int)(threadIdx.x & 63) * Op::kEpl};
+    typename Op::Raw raw;
     // workgroup-uniform choice of the access mode
     if (aligned) {
         if (base + Span<Op>::kElems <= t.n) {
-#pragma unroll
-            for (int i = 0; i < kPerWave; ++i) Op::template load<kVector>(t, first0 + i * kStride, raw[i]);
+            Op::template load<kVector>(t, first, raw);
             between();
-#pragma unroll
-            for (int i = 0; i < kPerWave; ++i) Op::template finish<kVector>(t, first0 + i * kStride, raw[i], h, lut_lane);
+            Op::template finish<kVector>(t, first, raw, h, lut);
         } else {
-#pragma unroll
-            for (int i = 0; i < kPerWave; ++i) Op::template load<kLane>(t, first0 + i * kStride, raw[i]);
+            Op::template load<kLane>(t, first, raw);
             between();
-#pragma unroll
-            for (int i = 0; i < kPerWave; ++i) Op::template finish<kLane>(t, first0 + i * kStride, raw[i], h, lut_lane);
+            Op::template finish<kLane>(t, first, raw, h, lut);
         }
     } else {
         between();
-#pragma unroll 1
-        for (int i = 0; i < kPerWave; ++i) {
-            Op::template load<kGuarded>(t, first0 + i * kStride, raw[0]);
-            Op::template finish<kGuarded>(t, first0 + i * kStride, raw[0], h, lut_lane);
-        }
+        Op::template load<kGuarded>(t, first, raw);
+        Op::template finish<kGuarded>(t, first, raw, h, lut);
     }
 }
 
-// Commits the first-moment table to LDS once per workgroup, at the first call.
-template <bool NEEDED> struct LutCommit {
-    float* lut; StepLut::Frag frag; bool done;
+// Commits the code tables to LDS once per workgroup, at the first call.
+template <int TABLES> struct LutCommit {
+    float* lut; typename StepLut<TABLES>::Frag frag; bool done;
     __device__ __forceinline__ void operator()() {
-        if constexpr (NEEDED) {
-            if (!done) { StepLut::commit(lut, frag); done = true; }
+        if constexpr (TABLES > 0) {
+            if (!done) { StepLut<TABLES>::commit(lut, frag); done = true; }
         }
     }
 };
 
 template <class Op>
 __global__ __launch_bounds__(kBlockThreads) void step_single_kernel(TensorPtrs t, typename Op::Hyper h) {
-    __shared__ __align__(16) float lut[Op::kNeedsLut ? StepLut::kFloats : 4];
+    __shared__ __align__(16) float lut[StepLut<Op::kLutTables>::kFloats];
     const int64_t base = (int64_t)blockIdx.x * Span<Op>::kElems;
-    LutCommit<Op::kNeedsLut> commit{lut, {}, false};
-    if constexpr (Op::kNeedsLut) commit.frag = StepLut::fetch();
-    run_span<Op>(t, base, all_aligned16(t), h, StepLut::lane_base(lut), commit);
+    LutCommit<Op::kLutTables> commit{lut, {}, false};
+    if constexpr (Op::kLutTables > 0) commit.frag = StepLut<Op::kLutTables>::fetch(kStepTables<Op::kDtype>.v);
+    run_span<Op>(t, base, all_aligned16(t), h, lut, commit);
 }
 
 // Workgroup b works on chunk b / kPerTile and takes span b % kPerTile of each of the chunk's tiles.
 template <class Op>
 __global__ __launch_bounds__(kBlockThreads) void step_multi_kernel(const fo_tensor_desc* __restrict__ descs,
                                                                    const fo_chunk* __restrict__ chunks, typename Op::Hyper h) {
-    __shared__ __align__(16) float lut[Op::kNeedsLut ? StepLut::kFloats : 4];
+    __shared__ __align__(16) float lut[StepLut<Op::kLutTables>::kFloats];
     constexpr int kPerTile = Span<Op>::kPerTile;
     const unsigned b = blockIdx.x;
     const fo_chunk ck = chunks[b / kPerTile];
     const TensorPtrs t = load_desc(descs + ck.tensor);
-    LutCommit<Op::kNeedsLut> commit{lut, {}, false};
-    if constexpr (Op::kNeedsLut) commit.frag = StepLut::fetch();
-    const float* lut_lane = StepLut::lane_base(lut);
+    LutCommit<Op::kLutTables> commit{lut, {}, false};
+    if constexpr (Op::kLutTables > 0) commit.frag = StepLut<Op::kLutTables>::fetch(kStepTables<Op::kDtype>.v);
     const bool aligned = all_aligned16(t);
     const int64_t in_tile = (int64_t)(b % kPerTile) * Span<Op>::kElems;
     for (int i = 0; i < ck.n_tiles; ++i) {
         const int64_t base = ((int64_t)ck.first_tile + i) * kTileElems + in_tile;
-        if (base < t.n) run_span<Op>(t, base, aligned, h, lut_lane, commit);
+        if (base < t.n) run_span<Op>(t, base, aligned, h, lut, commit);
     }
 }
 
@@ -265,15 +238,57 @@ inline int validate_multi(const fo_tensor_desc* descs, int64_t n_tensors, const 
 
 
 // Streaming from HBM degrades when a compute unit keeps too many bytes in flight, and a step wavefront has
-// several KiB of loads outstanding.  Each kernel family therefore names the LDS footprint it wants per
-// workgroup (Op::kLdsBytes; a compute unit has 160 KiB, so 11008 bytes admit 14 workgroups) and the launch
-// requests the difference to the kernel's own table as unused dynamic LDS.  The values sit in the middle of the
-// measured plateaus, away from the residencies (13 and 16 for Adam) where throughput drops by 4-5 %.
-template <class Op> inline unsigned lds_pad_bytes() {
-    const int env = step_lds_pad_bytes();
-    if (env >= 0) return (unsigned)env;
-    constexpr int kStatic = Op::kNeedsLut ? fo::StepLut::kFloats * 4 : 16;
-    return Op::kLdsBytes > kStatic ? Op::kLdsBytes - kStatic : 0;
+// several KiB of loads outstanding.  Each kernel family therefore names the number of workgroups it wants
+// resident per compute unit (Op::kWorkgroupsPerCu, the middle of the plateau measured on MI355X) and the launch
+// requests enough unused dynamic LDS to cap the residency there.  The request is derived from the device's LDS
+// per compute unit and confirmed with the runtime's occupancy query, once per kernel and device.
+struct Residency {
+    int target = 0;    // workgroups per compute unit asked for
+    int achieved = 0;  // what the occupancy query reports with `dynamic_lds`
+    unsigned dynamic_lds = 0;
+};
+
+template <class Kernel>
+Residency plan_residency(Kernel kernel, int target, int static_lds) {
+    Residency r;
+    r.target = target;
+    int dev = 0, lds_per_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&lds_per_cu, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, dev) != hipSuccess || lds_per_cu <= 0)
+        return r;
+    auto query = [&](long bytes) {
+        int n = 0;
+        const long dyn = bytes > static_lds ? bytes - static_lds : 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, fo::kBlockThreads, (size_t)dyn) != hipSuccess) n = 0;
+        return n;
+    };
+    // half-way between the footprints that would admit target and target + 1 workgroups, so that neither the
+    // allocation granularity nor a few bytes of static LDS tip the count
+    long bytes = ((long)lds_per_cu / target + (long)lds_per_cu / (target + 1)) / 2 / 256 * 256;
+    int got = query(bytes);
+    for (int tries = 0; tries < 64 && got != target && got > 0; ++tries) {
+        bytes += got > target ? 256 : -256;
+        if (bytes <= static_lds) { bytes = static_lds; got = query(bytes); break; }
+        got = query(bytes);
+    }
+    r.achieved = got;
+    r.dynamic_lds = (unsigned)(bytes > static_lds ? bytes - static_lds : 0);
+    return r;
+}
+
+// Residency of kernel K for Op on the current device (planned at the first launch there).
+template <class Op, class Kernel> const Residency& residency_of(Kernel kernel) {
+    constexpr int kMaxDevices = 64;
+    static Residency cache[kMaxDevices];
+    static std::once_flag once[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+    std::call_once(once[dev], [&] {
+        const int forced = debug_workgroups_per_cu();
+        constexpr int kStatic = fo::StepLut<Op::kLutTables>::kFloats * 4;
+        cache[dev] = plan_residency(kernel, forced > 0 ? forced : Op::kWorkgroupsPerCu, kStatic);
+    });
+    return cache[dev];
 }
 
 template <class Op>
@@ -281,7 +296,8 @@ int launch_single(const fo::TensorPtrs& t, const typename Op::Hyper& h, hipStrea
     // one pass over the tensor, one short-lived workgroup per span
     const int64_t grid = (t.n + fo::Span<Op>::kElems - 1) / fo::Span<Op>::kElems;
     if (grid > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "tensor too large for one launch (%lld elements)", (long long)t.n);
-    hipLaunchKernelGGL(fo::step_single_kernel<Op>, dim3((unsigned)grid), dim3(fo::kBlockThreads), lds_pad_bytes<Op>(), stream, t, h);
+    const unsigned lds = residency_of<Op>(fo::step_single_kernel<Op>).dynamic_lds;
+    hipLaunchKernelGGL(fo::step_single_kernel<Op>, dim3((unsigned)grid), dim3(fo::kBlockThreads), lds, stream, t, h);
     return check_hip(hipGetLastError(), "step kernel launch");
 }
 
@@ -289,7 +305,8 @@ template <class Op>
 int launch_multi(const fo_tensor_desc* descs, const fo_chunk* chunks, int64_t n_chunks, const typename Op::Hyper& h, hipStream_t stream) {
     const int64_t grid = n_chunks * fo::Span<Op>::kPerTile;
     if (grid > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "chunk table too large for one launch (%lld chunks)", (long long)n_chunks);
-    hipLaunchKernelGGL(fo::step_multi_kernel<Op>, dim3((unsigned)grid), dim3(fo::kBlockThreads), lds_pad_bytes<Op>(), stream, descs, chunks, h);
+    const unsigned lds = residency_of<Op>(fo::step_multi_kernel<Op>).dynamic_lds;
+    hipLaunchKernelGGL(fo::step_multi_kernel<Op>, dim3((unsigned)grid), dim3(fo::kBlockThreads), lds, stream, descs, chunks, h);
     return check_hip(hipGetLastError(), "multi-tensor step kernel launch");
 }
 

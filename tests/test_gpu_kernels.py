@@ -156,41 +156,49 @@ class _Case:
             else:
                 s.plain.copy_(a.cpu())
 
-    def compare(self, what, info):
-        """`info`: the oracle's intermediates of the step just taken."""
-        parity.check_master(self.gp, self.gecc, self.p, self.ecc, what,
-                            step_size=info["update_scale"])
-        stats = []
+    def compare(self, what, info, exact):
+        """`info`: the oracle's intermediates of the step just taken.  exact: every output bit must equal the
+        oracle's (all kernels but Adam on bf16 / fp16 parameters, see tests/parity.py).
+        Returns (worst code mismatch fraction, fraction of master weights beyond one unit with no allowance)."""
+        if exact:
+            assert parity.bits_equal(self.gp, self.p), f"{what}: parameter bits differ"
+            if self.ecc is not None:
+                assert parity.bits_equal(self.gecc, self.ecc), f"{what}: ECC bits differ"
+            for i, (s, (a, b)) in enumerate(zip(self.states, self.gstates)):
+                if self.quantized:
+                    assert parity.bits_equal(a, s.codes), f"{what} state{i}: codes differ"
+                    assert parity.bits_equal(b, s.scales), f"{what} state{i}: scales differ"
+                else:
+                    assert parity.bits_equal(a, s.plain), f"{what} state{i}: values differ"
+            return 0.0, 0.0
+        _, beyond = parity.check_master(self.gp, self.gecc, self.p, self.ecc, what, step_size=info["update_scale"])
+        worst = 0.0
         for i, (s, (a, b)) in enumerate(zip(self.states, self.gstates)):
             if self.quantized:
-                band = parity.near_tie_mom(info["m"]) if i == 0 else parity.near_tie_var(info["v"])
-                stats.append(parity.check_codes(a, s.codes, f"{what} state{i}", near_tie=band))
+                worst = max(worst, parity.check_codes(a, s.codes, f"{what} state{i}"))
                 parity.check_scales(b, s.scales, f"{what} state{i}")
             else:
-                got = a.cpu()
-                agree = (got == s.plain) | (torch.isnan(got) & torch.isnan(s.plain))  # same infinity / both NaN
-                d = (got.double() - s.plain.double()).abs()
-                assert bool((agree | (d <= parity.ulp_of(s.plain) * 1.0000001)).all()), f"{what} state{i}: more than one ulp"
-        return stats
+                assert parity.bits_equal(a, s.plain), f"{what} state{i}: unquantised state differs"
+        return worst, beyond
 
 
 def _adam_steps(n, dtype, ecc_dtype, quantized, decoupled, steps, seed, offset=0, grad_scale=1e-3):
+    """Returns per step (code mismatch fraction, fraction of master weights beyond one unit)."""
     k = _k()
     c = _Case(n, dtype, ecc_dtype, quantized, 2, seed, offset)
     lr, b1, b2, eps = 1e-3, 0.9, 0.999, 1e-8
     wd = 0.01 * lr if decoupled else 0.01
-    worst_raw = worst_filtered = 0.0
+    exact = dtype == torch.float32  # fp32 parameters: the update follows the reference operation by operation
+    out = []
     for step in range(1, steps + 1):
         g = _rand(n, grad_scale, 1000 * seed + step).to(dtype)
         gg = c._dev(g)
         (m, ms), (v, vs) = c.gstates
         k._fused_adam_step(m, ms, v, vs, c.gp, gg, c.gecc, lr, b1, b2, eps, wd, decoupled, step, quantize_optim_states=quantized)
         info = T.adam_step_ref(c.states[0], c.states[1], c.p, g, c.ecc, lr, b1, b2, eps, wd, decoupled, step)
-        stats = c.compare(f"adam n={n} {dtype} ecc={ecc_dtype} q={quantized} step={step}", info)
-        for raw, filt in stats:
-            worst_raw, worst_filtered = max(worst_raw, raw), max(worst_filtered, filt)
+        out.append(c.compare(f"adam n={n} {dtype} ecc={ecc_dtype} q={quantized} step={step}", info, exact))
         c.resync_oracle()
-    return worst_raw, worst_filtered
+    return out
 
 
 @pytest.mark.parametrize("dtype,ecc_dtype", VARIANTS)
@@ -198,16 +206,22 @@ def _adam_steps(n, dtype, ecc_dtype, quantized, decoupled, steps, seed, offset=0
 @pytest.mark.parametrize("decoupled", [True, False])
 def test_adam_step_matches_oracle(dtype, ecc_dtype, quantized, decoupled):
     for i, n in enumerate([1, 31, 33, 1000, 4096, 4097 + 4096, (1 << 16) + 17]):
-        _adam_steps(n, dtype, ecc_dtype, quantized, decoupled, steps=4, seed=i + 1)
+        stats = _adam_steps(n, dtype, ecc_dtype, quantized, decoupled, steps=4, seed=i + 1)
+        # the first step starts from zero states: m and v are formed exactly as the reference forms them and the
+        # requantiser follows its rounding, so not a single code may differ
+        assert stats[0][0] == 0.0, f"first-step codes differ (n={n})"
 
 
-def test_adam_headline_config_code_mismatch_rate():
-    """bf16 + int8 ECC + quantised AdamW on 2^20 and 2^20+17 elements, 10 steps: the sizes used for the
-    parity sub-check of the 2^30 throughput run."""
+@pytest.mark.parametrize("ecc_dtype", [torch.int8, torch.int16])
+def test_adam_headline_config_code_mismatch_rate(ecc_dtype):
+    """bf16 + ECC + quantised AdamW on 2^20 and 2^20+17 elements, 10 steps (the sizes of the parity sub-check of
+    the 2^30 throughput run): the raw mismatch rate of the codes on every step, the first included."""
     for n in [1 << 20, (1 << 20) + 17]:
-        raw, filtered = _adam_steps(n, torch.bfloat16, torch.int8, True, True, steps=10, seed=5)
-        print(f"n={n}: worst per-step code mismatch fraction raw {raw:.3e}, outside the tie band {filtered:.3e}")
-        assert filtered < parity.CODE_MISMATCH_FRACTION
+        stats = _adam_steps(n, torch.bfloat16, ecc_dtype, True, True, steps=10, seed=5)
+        print(f"n={n} ecc={ecc_dtype}: code mismatch per step " + " ".join(f"{a:.1e}" for a, _ in stats)
+              + "; master weights beyond one unit (no allowance) " + " ".join(f"{b:.1e}" for _, b in stats))
+        assert stats[0][0] == 0.0
+        assert max(a for a, _ in stats) < parity.CODE_MISMATCH_FRACTION
 
 
 def test_adam_unaligned_pointers():
@@ -243,7 +257,7 @@ def test_momentum_step_matches_oracle(dtype, ecc_dtype, quantized, mode):
             (m, ms), = c.gstates
             k._fused_momentum_step(m, ms, c.gp, g.to(DEV), c.gecc, quantize_optim_states=quantized, **kw)
             info = T.momentum_step_ref(c.states[0], c.p, g, c.ecc, **kw)
-            c.compare(f"{mode} n={n} {dtype} ecc={ecc_dtype} q={quantized} step={step}", info)
+            c.compare(f"{mode} n={n} {dtype} ecc={ecc_dtype} q={quantized} step={step}", info, exact=True)
             c.resync_oracle()
 
 
@@ -257,7 +271,7 @@ def test_plain_sgd_matches_oracle(dtype, ecc_dtype, decoupled, wd):
             g = _rand(n, 1e-2, 99 * i + step).to(dtype)
             k._sgd_plain_step(c.gp, g.to(DEV), c.gecc, 1e-2, wd, decoupled)
             info = T.momentum_step_ref(None, c.p, g, c.ecc, 1e-2, 0.0, 1.0, wd, decoupled=decoupled)
-            c.compare(f"plain sgd n={n} step={step}", info)
+            c.compare(f"plain sgd n={n} step={step}", info, exact=True)
             c.resync_oracle()
 
 
@@ -416,7 +430,7 @@ def test_randomised_configurations_match_oracle():
                 (m, ms), = c.gstates
                 k._fused_momentum_step(m, ms, c.gp, gg, c.gecc, quantize_optim_states=quantized, **kw)
                 info = T.momentum_step_ref(c.states[0], c.p, g, c.ecc, **kw)
-            c.compare(f"{what} step={step}", info)
+            c.compare(f"{what} step={step}", info, exact=kind != "adam" or dtype == torch.float32)
             c.resync_oracle()
 
 
