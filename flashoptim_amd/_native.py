@@ -66,6 +66,7 @@ SIGNATURES = {
     "fo_count_chunks": (_i64, [_vp, _i64, _i32]),
     "fo_build_chunks": (_i64, [_vp, _i64, _i32, _vp, _i64]),
     "fo_multi_adam_step": (_i32, [_vp, _i64, _vp, _i64, _i32, _i32, _i32] + [_f32] * 5 + [_i32, _i32, _vp]),
+    "fo_multi_adam_step_static": (_i32, [_vp, _i64, _i32, _i32, _i32] + [_f32] * 5 + [_i32, _i32, _vp]),
     "fo_multi_momentum_step": (_i32, [_vp, _i64, _vp, _i64, _i32, _i32, _i32] + [_f32] * 4 + [_i32, _i32, _i32, _vp]),
     "fo_multi_sgd_plain_step": (_i32, [_vp, _i64, _vp, _i64, _i32, _i32, _f32, _f32, _i32, _vp]),
     "fo_multi_absmax": (_i32, [_vp, _i64, _vp, _i64, _i32, _vp, _vp]),

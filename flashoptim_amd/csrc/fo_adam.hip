@@ -2,6 +2,8 @@
 // optimizers.py:2203-2438, cited as "ref:").
 #include "fo_step.h"
 
+#include <mutex>
+
 namespace fo {
 
 // What a lane holds between issuing its loads and consuming them.
@@ -128,6 +130,64 @@ template <int DT, int EB, bool Q> using AdamWOp = fo::AdamOp<DT, EB, Q, true>;  
 
 using fo::make_adam_hyper;
 
+// ------------------------------------------------------------------------------------------------
+// launch tables held in a static device array (fo_multi_adam_step_static)
+// ------------------------------------------------------------------------------------------------
+// Layout of the array: kStaticMaxTensors descriptors, then kStaticMaxChunks chunk entries.  Every device the
+// library runs on holds its own copy until the process ends (1.06 MiB).  Calls on one device share it and keep
+// the previous call's tables; a call overwrites every entry it uses, so nothing has to be cleared.
+constexpr int64_t kStaticMaxTensors = FO_STATIC_MAX_TENSORS;
+constexpr int64_t kStaticMaxChunks = FO_STATIC_MAX_CHUNKS;
+constexpr size_t kStaticBytes = kStaticMaxTensors * sizeof(fo_tensor_desc) + kStaticMaxChunks * sizeof(fo_chunk);
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kStaticBytes];
+
+// Device address of `scratch` on the current device.  The array's name is only a host-side handle: the address a
+// kernel can use comes from hipGetSymbolAddress, once per device, with that device current.
+int static_tables(int* device_out, fo_tensor_desc** descs, fo_chunk** chunks) {
+    constexpr int kMaxDevices = 64;
+    static void* base[kMaxDevices];
+    static std::once_flag once[kMaxDevices];
+    static hipError_t status[kMaxDevices];
+    int dev = 0;
+    if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    if (dev < 0 || dev >= kMaxDevices) return fail(FO_ERR_NO_DEVICE, "device index %d out of range", dev);
+    std::call_once(once[dev], [&] { status[dev] = hipGetSymbolAddress(&base[dev], HIP_SYMBOL(scratch)); });
+    if (int rc = check_hip(status[dev], "hipGetSymbolAddress(scratch)")) return rc;
+    if (!base[dev]) return fail(FO_ERR_NO_DEVICE, "static table array has no device address");
+    *device_out = dev;
+    *descs = reinterpret_cast<fo_tensor_desc*>(base[dev]);
+    *chunks = reinterpret_cast<fo_chunk*>(static_cast<unsigned char*>(base[dev]) + kStaticMaxTensors * sizeof(fo_tensor_desc));
+    return 0;
+}
+
+// A batch of descriptors travels to the device as a kernel argument (no copy engine, no staging memory):
+// workgroup i of the launch writes descriptor i of the batch and the chunk entries of that tensor.
+constexpr int kStageBatch = 48;
+struct StageBatch {
+    fo_tensor_desc desc[kStageBatch];
+    int32_t first_chunk[kStageBatch];
+    int32_t base_tensor, count, tiles_per_chunk, reserved;
+};
+static_assert(sizeof(StageBatch) <= 3584, "a batch must fit the kernel argument segment");
+
+__global__ __launch_bounds__(256) void stage_tables_kernel(StageBatch b, fo_tensor_desc* descs, fo_chunk* chunks) {
+    const int i = blockIdx.x;
+    if (i >= b.count) return;
+    const int tensor = b.base_tensor + i;
+    if (threadIdx.x == 0) descs[tensor] = b.desc[i];
+    const int64_t tiles = (b.desc[i].n + fo::kTileElems - 1) / fo::kTileElems;
+    const int64_t n_chunks = (tiles + b.tiles_per_chunk - 1) / b.tiles_per_chunk;
+    for (int64_t c = threadIdx.x; c < n_chunks; c += blockDim.x) {
+        fo_chunk ck;
+        ck.tensor = tensor;
+        ck.first_tile = (int32_t)(c * b.tiles_per_chunk);
+        const int64_t left = tiles - c * b.tiles_per_chunk;
+        ck.n_tiles = (int32_t)(left < b.tiles_per_chunk ? left : b.tiles_per_chunk);
+        ck.reserved = 0;
+        chunks[b.first_chunk[i] + c] = ck;
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -152,6 +212,69 @@ int fo_multi_adam_step(const fo_tensor_desc* descs, int64_t n_tensors, const fo_
     if (n_chunks == 0) return 0;
     if (step < 1) return fail(FO_ERR_INVALID_ARGUMENT, "step must be >= 1 (got %d)", step);
     MultiLauncher<fo::AdamHyper> L{descs, chunks, n_chunks, make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step), (hipStream_t)stream};
+    return decoupled ? dispatch<AdamWOp>(dtype, ecc_bytes, quantized, L) : dispatch<AdamL2Op>(dtype, ecc_bytes, quantized, L);
+}
+
+int fo_multi_adam_step_static(const fo_tensor_desc* host_descs, int64_t n_tensors, int dtype, int ecc_bytes, int quantized,
+                              float lr, float beta1, float beta2, float eps, float weight_decay, int decoupled, int step,
+                              void* stream) {
+    if (n_tensors < 0) return fail(FO_ERR_INVALID_ARGUMENT, "negative tensor count");
+    if (n_tensors > kStaticMaxTensors)
+        return fail(FO_ERR_INVALID_ARGUMENT, "%lld tensors exceed the static table's %lld (use fo_multi_adam_step with caller-owned tables)",
+                    (long long)n_tensors, (long long)kStaticMaxTensors);
+    if (n_tensors > 0 && !host_descs) return fail(FO_ERR_INVALID_ARGUMENT, "host_descs must not be NULL");
+    if (dtype < FO_F32 || dtype > FO_F16) return fail(FO_ERR_INVALID_ARGUMENT, "unknown dtype %d", dtype);
+    if (ecc_bytes < 0 || ecc_bytes > 2) return fail(FO_ERR_INVALID_ARGUMENT, "ecc_bytes must be 0, 1 or 2 (got %d)", ecc_bytes);
+    if (dtype == FO_F32 && ecc_bytes != 0) return fail(FO_ERR_UNSUPPORTED, "fp32 parameters carry no ECC");
+    if (step < 1) return fail(FO_ERR_INVALID_ARGUMENT, "step must be >= 1 (got %d)", step);
+    int64_t total_tiles = 0;
+    for (int64_t i = 0; i < n_tensors; ++i) {
+        const fo_tensor_desc& d = host_descs[i];
+        if (d.n < 0) return fail(FO_ERR_INVALID_ARGUMENT, "tensor %lld has negative length", (long long)i);
+        if (d.n == 0) continue;
+        if (int rc = validate_common(d.param, d.grad, d.ecc, d.n, dtype, ecc_bytes)) return rc;
+        if (int rc = validate_state(d.mom, d.mom_scales, quantized, dtype, "mom")) return rc;
+        if (int rc = validate_state(d.var, d.var_scales, quantized, dtype, "var")) return rc;
+        const int64_t tiles = (d.n + fo::kTileElems - 1) / fo::kTileElems;
+        if (tiles > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "tensor %lld too large", (long long)i);
+        total_tiles += tiles;
+    }
+    if (total_tiles == 0) return 0;
+    // the fewest tiles per chunk that keep the chunk table inside the array (every tensor may end with a short chunk)
+    int64_t tiles_per_chunk = 1;
+    auto count_chunks = [&](int64_t tpc) {
+        int64_t c = 0;
+        for (int64_t i = 0; i < n_tensors; ++i) c += ((host_descs[i].n + fo::kTileElems - 1) / fo::kTileElems + tpc - 1) / tpc;
+        return c;
+    };
+    int64_t n_chunks = count_chunks(tiles_per_chunk);
+    if (n_chunks > kStaticMaxChunks) {  // count <= total_tiles / tpc + n_tensors
+        tiles_per_chunk = (total_tiles + (kStaticMaxChunks - n_tensors) - 1) / (kStaticMaxChunks - n_tensors);
+        if (tiles_per_chunk > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "tensor list too large for the static chunk table");
+        n_chunks = count_chunks(tiles_per_chunk);
+    }
+    int dev = 0;
+    fo_tensor_desc* d_descs = nullptr;
+    fo_chunk* d_chunks = nullptr;
+    if (int rc = static_tables(&dev, &d_descs, &d_chunks)) return rc;
+
+    StageBatch b;
+    int64_t next_chunk = 0;
+    for (int64_t t0 = 0; t0 < n_tensors; t0 += kStageBatch) {
+        b.base_tensor = (int32_t)t0;
+        b.count = (int32_t)((n_tensors - t0) < kStageBatch ? (n_tensors - t0) : kStageBatch);
+        b.tiles_per_chunk = (int32_t)tiles_per_chunk;
+        b.reserved = 0;
+        for (int i = 0; i < b.count; ++i) {
+            b.desc[i] = host_descs[t0 + i];
+            b.first_chunk[i] = (int32_t)next_chunk;
+            const int64_t tiles = (b.desc[i].n + fo::kTileElems - 1) / fo::kTileElems;
+            next_chunk += (tiles + tiles_per_chunk - 1) / tiles_per_chunk;
+        }
+        hipLaunchKernelGGL(stage_tables_kernel, dim3((unsigned)b.count), dim3(256), 0, (hipStream_t)stream, b, d_descs, d_chunks);
+        if (int rc = check_hip(hipGetLastError(), "table staging kernel launch")) return rc;
+    }
+    MultiLauncher<fo::AdamHyper> L{d_descs, d_chunks, n_chunks, make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step), (hipStream_t)stream};
     return decoupled ? dispatch<AdamWOp>(dtype, ecc_bytes, quantized, L) : dispatch<AdamL2Op>(dtype, ecc_bytes, quantized, L);
 }
 

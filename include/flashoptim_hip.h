@@ -120,6 +120,23 @@ int fo_multi_momentum_step(const fo_tensor_desc *descs, int64_t n_tensors, const
                            float update_coef, float weight_decay, int decoupled, int nesterov, int do_lion,
                            void *stream);
 
+/*
+ * fo_multi_adam_step for callers that cannot allocate device memory or copy tables to it (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The caller passes the descriptors as a HOST array; the library keeps the descriptor and chunk tables in a static
+ * device array of its own (FO_STATIC_MAX_TENSORS descriptors + FO_STATIC_MAX_CHUNKS chunk entries, 1.06 MiB per
+ * device, held until the process ends), fills them with small kernels whose arguments carry the descriptors, and
+ * launches the same step kernel.  It calls no hipMalloc / hipFree / hipMemcpy.  Lists with more than
+ * FO_STATIC_MAX_TENSORS tensors are refused; lists with more than FO_STATIC_MAX_CHUNKS tiles are covered with
+ * several 4096-element tiles per work item.  Results are bit-identical to fo_multi_adam_step.  All calls on one
+ * device share the one array: calls that overlap in time on a device (different streams or threads) race.
+ */
+#define FO_STATIC_MAX_TENSORS 1024
+#define FO_STATIC_MAX_CHUNKS 65536
+int fo_multi_adam_step_static(const fo_tensor_desc *host_descs, int64_t n_tensors, int dtype, int ecc_bytes,
+                              int quantized, float lr, float beta1, float beta2, float eps, float weight_decay,
+                              int decoupled, int step, void *stream);
+
 /* Momentum-free SGD over many tensors: the multi-tensor form of fo_sgd_plain_step (descs use param, grad, ecc, n). */
 int fo_multi_sgd_plain_step(const fo_tensor_desc *descs, int64_t n_tensors, const fo_chunk *chunks,
                             int64_t n_chunks, int dtype, int ecc_bytes, float lr, float weight_decay,
