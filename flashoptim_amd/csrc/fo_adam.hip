@@ -85,8 +85,12 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
         // group absmax (ref:2399-2404)
         am = fmaxf(group_max<EPL>(am), 1e-12f);
         av = fmaxf(group_max<EPL>(av), 1e-12f);
-        quantize_mom<EPL>(m, am, raw.m);
-        quantize_var<EPL>(r, av, raw.v);
+        if constexpr (EPL == 8) {
+            quantize_mom<EPL>(m, am, raw.m);
+            quantize_var<EPL>(r, av, raw.v);
+        } else {
+            quantize_mom_var(m, am, r, av, raw.m, raw.v);
+        }
         store_lane<1, EPL, FAST>(raw.m, t.mom, w, n);
         store_lane<1, EPL, FAST>(raw.v, t.var, w, n);
         if (live_group && (threadIdx.x & (32 / EPL - 1)) == 0) {                    // ref:2424-2434

@@ -273,6 +273,40 @@ template <int EB, int EPL> __device__ __forceinline__ void pack_codes(const u32 
     }
 }
 
+// Converts eight floats to integers and packs the low byte of each into two dwords: a[0..3] -> lo, b[0..3] -> hi.
+// KIND_A / KIND_B: kFloor = (int)floor(x) (signed first-moment codes), kTrunc = truncation (non-negative
+// second-moment codes).  Each conversion writes its byte straight into the destination dword (sub-dword
+// destination select), so no separate packing instructions are needed.
+// The hazard recogniser does not look inside asm: on gfx940/gfx950 a VALU instruction that reads a register
+// written by the preceding instruction with a sub-dword destination select needs one wait state, and a byte write
+// that preserves the rest of the dword reads it.  The two chains are therefore interleaved (every dependent pair
+// has an independent instruction between it) and the block ends with a wait state for whatever reads the result.
+enum { kFloor = 0, kTrunc = 1 };
+#define FO_CVT_FLOOR "v_cvt_flr_i32_f32_sdwa"
+#define FO_CVT_TRUNC "v_cvt_i32_f32_sdwa"
+#define FO_CONVERT_PACK8(OPA, OPB)                                                                          \
+    asm(OPA " %0, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"                               \
+        OPB " %1, %6 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"                               \
+        OPA " %0, %3 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"                          \
+        OPB " %1, %7 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"                          \
+        OPA " %0, %4 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"                          \
+        OPB " %1, %8 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"                          \
+        OPA " %0, %5 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"                          \
+        OPB " %1, %9 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"                          \
+        "s_nop 0"                                                                                           \
+        : "=&v"(lo), "=&v"(hi)                                                                              \
+        : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]))
+template <int KIND_A, int KIND_B>
+__device__ __forceinline__ void convert_pack8(const float (&a)[4], const float (&b)[4], u32& lo, u32& hi) {
+    if constexpr (KIND_A == kFloor && KIND_B == kFloor) FO_CONVERT_PACK8(FO_CVT_FLOOR, FO_CVT_FLOOR);
+    else if constexpr (KIND_A == kTrunc && KIND_B == kTrunc) FO_CONVERT_PACK8(FO_CVT_TRUNC, FO_CVT_TRUNC);
+    else if constexpr (KIND_A == kFloor && KIND_B == kTrunc) FO_CONVERT_PACK8(FO_CVT_FLOOR, FO_CVT_TRUNC);
+    else FO_CONVERT_PACK8(FO_CVT_TRUNC, FO_CVT_FLOOR);
+}
+#undef FO_CONVERT_PACK8
+#undef FO_CVT_FLOOR
+#undef FO_CVT_TRUNC
+
 // ------------------------------------------------------------------------------------------------
 // 8-bit group codec pieces used by the fused kernels
 // ------------------------------------------------------------------------------------------------

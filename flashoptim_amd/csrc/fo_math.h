@@ -208,16 +208,20 @@ typedef StepTables<DT_BF16> SoftsignTable;  // first 256 entries: the same for e
 // floor is taken of the rounded sum.  Doubling is exact, so RN(2nm / d) * 127 is formed as RN(nm / d) * 254.
 // ram / rav: the reciprocal instruction applied to the group absmax (shared by the lanes of the group).
 // Returns a word whose low byte is the code.
-FO_FN u32 quantize_mom_code(float m, float am, float ram) {
+// The *_rounded functions return the rounded sum fl(x + 0.5) whose floor is the code (the kernels convert and pack
+// four of them at a time); the *_code functions finish the job for one value.
+FO_FN float quantize_mom_rounded(float m, float am, float ram) {
     const float nm = div_corrected(m, am, ram);
     const float d = 1.0f + fabsf(nm);
     const float t = div_corrected(nm, d, hw::rcp(d));
-    return (u32)hw::floor_to_int(t * 254.0f + 0.5f);
+    return t * 254.0f + 0.5f;
 }
-FO_FN u32 quantize_var_code(float r, float av, float rav) {
+FO_FN float quantize_var_rounded(float r, float av, float rav) {
     const float q = div_corrected(r, av, rav);
-    return (u32)(int)(q * 255.0f + 0.5f);  // non-negative: truncation is the floor
+    return q * 255.0f + 0.5f;  // non-negative: truncation is the floor
 }
+FO_FN u32 quantize_mom_code(float m, float am, float ram) { return (u32)hw::floor_to_int(quantize_mom_rounded(m, am, ram)); }
+FO_FN u32 quantize_var_code(float r, float av, float rav) { return (u32)(int)quantize_var_rounded(r, av, rav); }
 
 // ------------------------------------------------------------------------------------------------
 // Adam / AdamW element update (ref:2296-2375)

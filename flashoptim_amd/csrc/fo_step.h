@@ -86,22 +86,50 @@ __device__ __forceinline__ void write_master(const float (&p)[EPL], Pack<DTypeIn
 
 // Quantises the lane's first-moment values against the group absmax `am` (shared by the group's lanes, clamped
 // at 1e-12) and the lane's sqrt(v) values against the group maximum `av`; the rounding is the reference's
-// (fo_math.h: quantize_mom_code, quantize_var_code; ref:2405-2419, 1703-1710).
+// (fo_math.h: quantize_mom_rounded, quantize_var_rounded; ref:2405-2419, 1703-1710).
 template <int EPL>
 __device__ __forceinline__ void quantize_mom(const float (&m)[EPL], float am, Pack<1, EPL>& out) {
+    static_assert(EPL == 8, "two dwords of codes per lane");
     const float ram = hw::rcp(am);
-    u32 b[EPL];
+    float lo[4], hi[4];
 #pragma unroll
-    for (int k = 0; k < EPL; ++k) b[k] = quantize_mom_code(m[k], am, ram);
-    pack_codes<1, EPL>(b, out);
+    for (int k = 0; k < 4; ++k) {
+        lo[k] = quantize_mom_rounded(m[k], am, ram);
+        hi[k] = quantize_mom_rounded(m[k + 4], am, ram);
+    }
+    convert_pack8<kFloor, kFloor>(lo, hi, out.w[0], out.w[1]);
 }
 template <int EPL>
 __device__ __forceinline__ void quantize_var(const float (&r)[EPL], float av, Pack<1, EPL>& out) {
+    static_assert(EPL == 8, "two dwords of codes per lane");
     const float rav = hw::rcp(av);
-    u32 b[EPL];
+    float lo[4], hi[4];
 #pragma unroll
-    for (int k = 0; k < EPL; ++k) b[k] = quantize_var_code(r[k], av, rav);
-    pack_codes<1, EPL>(b, out);
+    for (int k = 0; k < 4; ++k) {
+        lo[k] = quantize_var_rounded(r[k], av, rav);
+        hi[k] = quantize_var_rounded(r[k + 4], av, rav);
+    }
+    convert_pack8<kTrunc, kTrunc>(lo, hi, out.w[0], out.w[1]);
+}
+// Four elements per lane (fp32 parameters): one dword of codes per state; the two states share the conversion block.
+__device__ __forceinline__ void quantize_mom_var(const float (&m)[4], float am, const float (&r)[4], float av,
+                                                 Pack<1, 4>& mout, Pack<1, 4>& vout) {
+    const float ram = hw::rcp(am), rav = hw::rcp(av);
+    float a[4], b[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        a[k] = quantize_mom_rounded(m[k], am, ram);
+        b[k] = quantize_var_rounded(r[k], av, rav);
+    }
+    convert_pack8<kFloor, kTrunc>(a, b, mout.w[0], vout.w[0]);
+}
+// Four elements per lane, one state (momentum kernels on fp32 parameters): plain conversion and byte packing.
+__device__ __forceinline__ void quantize_mom(const float (&m)[4], float am, Pack<1, 4>& out) {
+    const float ram = hw::rcp(am);
+    u32 b[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) b[k] = quantize_mom_code(m[k], am, ram);
+    pack_codes<1, 4>(b, out);
 }
 
 template <int DT, int EPL>
