@@ -74,7 +74,10 @@ SIGNATURES = {
     "fo_dequantize": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp]),
     "fo_ecc_join": (_i32, [_vp, _i32, _vp, _i32, _vp, _i64, _vp]),
     "fo_ecc_split": (_i32, [_vp, _vp, _i32, _vp, _i32, _i64, _vp]),
+    # include/flashoptim_hip_diag.h
     "fo_copy_bytes": (_i32, [_vp, _vp, _i64, _vp]),
+    "fo_adam_step_residency": (_i32, [_i32] * 5 + [_vp] * 3),
+    "fo_momentum_step_residency": (_i32, [_i32] * 5 + [_vp] * 3),
 }
 
 

@@ -73,6 +73,7 @@ class _Bucket:
     plan: Optional[BucketPlan]        # multi-tensor tables; None for single-tensor buckets
     step_pool: Optional[torch.Tensor]  # 1-D CPU fp32 tensor whose elements ARE the bucket's `step` scalars (Adam), else None
     step_value: Optional[int]
+    step_views: Optional[list] = None  # the 0-dim views of step_pool that were stored as state[p]["step"]
 
 
 @dataclass
@@ -401,6 +402,13 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
     def _step_group_slow(self, index: int, group: dict[str, Any]) -> None:
         """Full per-parameter planning (state creation, checks, counters), then one launch per bucket; leaves a
         cache behind that stays valid while the same parameters have gradients (frozen or unused ones sit out)."""
+        if torch.cuda.is_current_stream_capturing() and self._group_cache.get(index) is not None:
+            # a cached group fell back to full planning (a parameter, gradient layout or hyper-parameter changed):
+            # that builds new launch tables, which a HIP graph cannot record
+            raise RuntimeError(
+                "step() has to re-plan its launches (a gradient is missing or has a new layout, a parameter was "
+                "replaced, or a counter was rewritten), which cannot be recorded into a HIP graph. Run one step "
+                "outside the capture with the tensors the graph will use, then capture.")
         planned: dict[LaunchKey, list] = {}
         cacheable = True
         idle = []
@@ -430,17 +438,18 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
             else:
                 for t in tensors:
                     self._launch_single(key, t)
-            step_pool = None
+            step_pool, step_views = None, None
             if "step" in scalars:
                 # the per-parameter CPU `step` scalars become 0-dim views into one tensor, so that the cached path
                 # advances all of them with a single in-place add (one add per scalar costs 1.3 us each)
                 step_pool = torch.stack([self.state[p]["step"].detach().reshape(()) for p, _ in items])
-                for i, (p, _) in enumerate(items):
-                    self.state[p]["step"] = step_pool[i]
+                step_views = [step_pool[i] for i in range(len(items))]
+                for view, (p, _) in zip(step_views, items):
+                    self.state[p]["step"] = view
             for t in tensors:
                 t.grad = None  # the cache must not keep gradients alive
             buckets.append(_Bucket(key.kind, key.dtype, key.ecc_bytes, key.quantized, [p for p, _ in items], tensors,
-                                   plan, step_pool, scalars.get("step")))
+                                   plan, step_pool, scalars.get("step"), step_views))
         if cacheable and buckets:
             needed = None
             if self._check_numerics:
@@ -462,7 +471,12 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
         for b in cache.buckets:
             if b.step_pool is not None:
                 # the counters are live state the caller may have rewritten (a warm restart zeroes them): take the
-                # step number from them, and leave counters that no longer agree to the per-parameter path
+                # step number from them, and leave counters that no longer agree to the per-parameter path.  A
+                # counter OBJECT that was replaced (state[p]["step"] = tensor(0.)) no longer aliases the pool.
+                state = self.state
+                for p, view in zip(b.params, b.step_views):
+                    if state[p].get("step") is not view:
+                        return False
                 lo, hi = torch.aminmax(b.step_pool)
                 lo = lo.item()
                 if lo != hi.item():

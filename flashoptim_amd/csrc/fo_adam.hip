@@ -1,6 +1,7 @@
 // Fused Adam / AdamW step kernel for gfx950 and its C entry points (ref: /root/reference/flashoptim/
 // optimizers.py:2203-2438, cited as "ref:").
 #include "fo_step.h"
+#include "../../include/flashoptim_hip_diag.h"
 
 #include <mutex>
 
@@ -280,6 +281,12 @@ int fo_multi_adam_step_static(const fo_tensor_desc* host_descs, int64_t n_tensor
     }
     MultiLauncher<fo::AdamHyper> L{d_descs, d_chunks, n_chunks, make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step), (hipStream_t)stream};
     return decoupled ? dispatch<AdamWOp>(dtype, ecc_bytes, quantized, L) : dispatch<AdamL2Op>(dtype, ecc_bytes, quantized, L);
+}
+
+int fo_adam_step_residency(int dtype, int ecc_bytes, int quantized, int decoupled, int multi, int* target, int* achieved,
+                           int* dynamic_lds) {
+    ResidencyQuery q{multi, target, achieved, dynamic_lds};
+    return decoupled ? dispatch<AdamWOp>(dtype, ecc_bytes, quantized, q) : dispatch<AdamL2Op>(dtype, ecc_bytes, quantized, q);
 }
 
 }  // extern "C"

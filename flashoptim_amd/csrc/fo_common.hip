@@ -3,6 +3,7 @@
 #include "fo_device.h"
 #include "fo_host.h"
 #include "../../include/flashoptim_hip.h"
+#include "../../include/flashoptim_hip_diag.h"
 
 #include <cstdarg>
 #include <cstdio>

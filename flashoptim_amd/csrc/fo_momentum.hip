@@ -1,6 +1,7 @@
 // Fused SGD / SGDW / Nesterov / Lion step kernels (and the momentum-free SGD step) for gfx950 with their C
 // entry points (ref: /root/reference/flashoptim/optimizers.py:1447-1465, 1535-1719, cited as "ref:").
 #include "fo_step.h"
+#include "../../include/flashoptim_hip_diag.h"
 
 namespace fo {
 
@@ -145,6 +146,14 @@ int fo_multi_sgd_plain_step(const fo_tensor_desc* descs, int64_t n_tensors, cons
     if (n_chunks == 0) return 0;
     MultiLauncher<fo::MomentumHyper> L{descs, chunks, n_chunks, make_momentum_hyper(lr, 0.0f, 1.0f, weight_decay, decoupled, 0), (hipStream_t)stream};
     return dispatch<PlainOp>(dtype, ecc_bytes, 0, L);
+}
+
+int fo_momentum_step_residency(int dtype, int ecc_bytes, int quantized, int kind, int multi, int* target, int* achieved,
+                               int* dynamic_lds) {
+    ResidencyQuery q{multi, target, achieved, dynamic_lds};
+    if (kind == fo::KIND_LION) return dispatch<LionOp>(dtype, ecc_bytes, quantized, q);
+    if (kind == fo::KIND_PLAIN) return dispatch<PlainOp>(dtype, ecc_bytes, 0, q);
+    return dispatch<SgdOp>(dtype, ecc_bytes, quantized, q);
 }
 
 }  // extern "C"

@@ -353,6 +353,18 @@ int dispatch(int dtype, int ecc_bytes, int quantized, F&& f) {
     return fail(FO_ERR_UNSUPPORTED, "unsupported dtype/ecc combination (%d, %d)", dtype, ecc_bytes);
 }
 
+// Reports the residency plan of a kernel family (diagnostic entry points): 0 on success.
+struct ResidencyQuery {
+    int multi; int* target; int* achieved; int* dynamic_lds;
+    template <class Op> int operator()() {
+        const Residency& r = multi ? residency_of<Op>(fo::step_multi_kernel<Op>) : residency_of<Op>(fo::step_single_kernel<Op>);
+        if (target) *target = r.target;
+        if (achieved) *achieved = r.achieved;
+        if (dynamic_lds) *dynamic_lds = (int)r.dynamic_lds;
+        return r.achieved > 0 ? 0 : fail(FO_ERR_NO_DEVICE, "occupancy query failed");
+    }
+};
+
 template <class H> struct SingleLauncher {
     fo::TensorPtrs t; H h; hipStream_t s;
     template <class Op> int operator()() { return launch_single<Op>(t, h, s); }

@@ -9,9 +9,11 @@ hyper-parameters into a *bucket* and issues one launch per bucket.  A bucket own
 * the descriptor table (``fo_tensor_desc``: the raw pointers of every tensor).  Parameters and optimizer states
   keep their addresses; gradients are re-allocated by ``zero_grad(set_to_none=True)`` (although the caching
   allocator usually hands back the same addresses), so each step only compares gradient addresses and re-uploads
-  the table when one moved.  The upload goes through pinned host memory with a stream-ordered copy: ``step``
-  never synchronises with the device.  The table holds addresses, not tensor references, so a freed gradient
-  is not kept alive.
+  the table when one moved.  The upload goes through one pinned staging buffer per bucket with a stream-ordered
+  copy: ``step`` never waits for the device (it only waits for the previous upload of the same bucket to have left
+  the staging buffer, which has long happened).  The table holds addresses, not tensor references, so a freed
+  gradient is not kept alive.  Under HIP graph capture a table cannot be built or re-uploaded (the copy would be
+  recorded with the staging buffer's contents of that moment): ``launch`` raises instead, see there.
 
 Chunks never straddle tensors and start on 4096-element boundaries counted from element 0 of their tensor, so
 quantisation groups are exactly those of a per-tensor launch and the result is bit-identical to it.
@@ -127,9 +129,18 @@ class BucketPlan:
         self.grad_ptrs = [d.grad for d in self.table]
         self.param_ptrs = [d.param for d in self.table]
 
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(
+                "The launch tables of a multi-tensor step cannot be built while a HIP graph is being captured. Run one "
+                "step outside the capture first, with the gradient buffers the graph will use.")
         host, self.n_chunks = chunk_table(numels, tiles_per_chunk)
         self.chunks_dev = host.to(self.device)
-        self.descs_dev = torch.empty(self.n_tensors * ctypes.sizeof(FoTensorDesc), dtype=torch.uint8, device=self.device)
+        nbytes = self.n_tensors * ctypes.sizeof(FoTensorDesc)
+        self.descs_dev = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        # one pinned staging buffer for the life of the plan; `_staged` marks the last copy out of it
+        self._staging = torch.empty(nbytes, dtype=torch.uint8).pin_memory()
+        self._table_bytes = torch.frombuffer(self.table, dtype=torch.uint8)  # a view of the ctypes table, no copy
+        self._staged: Optional[torch.cuda.Event] = None
         self._dirty = True
 
     def set_grad_ptr(self, index: int, ptr: int) -> None:
@@ -138,10 +149,20 @@ class BucketPlan:
         self._dirty = True
 
     def _upload(self) -> None:
-        staged = torch.frombuffer(bytearray(bytes(self.table)), dtype=torch.uint8).pin_memory()
-        # stream-ordered: launches already queued with the previous table finish before it is overwritten; the
-        # pinned staging block is recycled by torch's host allocator only after the copy has run
-        self.descs_dev.copy_(staged, non_blocking=True)
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(
+                "A gradient of this multi-tensor step moved to another address, so its pointer table has to be "
+                "uploaded again, which cannot be recorded into a HIP graph (a replay would copy whatever the staging "
+                "buffer holds by then). Run one step outside the capture with the gradient buffers the graph will use "
+                "(static gradients, zero_grad(set_to_none=False)), then capture.")
+        if self._staged is not None:
+            self._staged.synchronize()  # the previous upload has read the staging buffer (normally long ago)
+        self._staging.copy_(self._table_bytes)
+        # stream-ordered: launches already queued with the previous table finish before it is overwritten
+        self.descs_dev.copy_(self._staging, non_blocking=True)
+        if self._staged is None:
+            self._staged = torch.cuda.Event()
+        self._staged.record()
         self._dirty = False
 
     def launch(self, **scalars) -> None:

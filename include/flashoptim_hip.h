@@ -173,13 +173,6 @@ int fo_ecc_join(const void *narrow, int narrow_dtype, const void *ecc, int ecc_b
 int fo_ecc_split(const float *x, const void *narrow, int narrow_dtype, void *ecc, int ecc_bytes, int64_t n,
                  void *stream);
 
-/*
- * Measurement aid: a plain device-to-device copy kernel (128-bit loads and stores, same launch geometry as
- * the step kernels) used to calibrate hardware byte counters and to show the attainable HBM rate next to the
- * step kernels.  n_bytes must be a multiple of 16 and both pointers 16-byte aligned.
- */
-int fo_copy_bytes(void *dst, const void *src, int64_t n_bytes, void *stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,38 @@
+/*
+ * flashoptim_hip_diag.h -- measurement and diagnostic entry points of libflashoptim_hip.so.
+ *
+ * Nothing here is part of the optimizer path and none of it has a counterpart in the reference
+ * (/root/reference/flashoptim/optimizers.py): the symbols exist for the benchmark and the tests.
+ */
+#ifndef FLASHOPTIM_HIP_DIAG_H
+#define FLASHOPTIM_HIP_DIAG_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * A plain device-to-device copy kernel (128-bit loads and stores, same launch geometry and store policy as the
+ * step kernels) used to calibrate hardware byte counters and to show the attainable HBM rate next to the step
+ * kernels.  n_bytes must be a multiple of 16 and both pointers 16-byte aligned.
+ */
+int fo_copy_bytes(void *dst, const void *src, int64_t n_bytes, void *stream);
+
+/*
+ * Residency plan of a step kernel on the current device: the workgroups per compute unit the kernel family asks
+ * for (`target`), what the runtime's occupancy query reports for the dynamic LDS request that enforces it
+ * (`achieved`) and that request in bytes (`dynamic_lds`).  Any output pointer may be NULL.
+ *   multi: 0 = the single-tensor kernel, 1 = the multi-tensor kernel.
+ *   kind (momentum): 0 = SGD / SGDW / Nesterov, 1 = Lion, 2 = momentum-free SGD.
+ */
+int fo_adam_step_residency(int dtype, int ecc_bytes, int quantized, int decoupled, int multi, int *target,
+                           int *achieved, int *dynamic_lds);
+int fo_momentum_step_residency(int dtype, int ecc_bytes, int quantized, int kind, int multi, int *target,
+                               int *achieved, int *dynamic_lds);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHOPTIM_HIP_DIAG_H */

@@ -14,6 +14,11 @@ MODES = [(True, False, False), (True, False, True), (False, False, False), (Fals
 SIZES = [1, 5, 31, 32, 33, 1000, 4095, 4096, 4097, 3 * 4096 + 555, 1 << 18]
 
 
+def _native_lib():
+    from flashoptim_amd import _native
+    return _native.lib()
+
+
 def _k():
     from flashoptim_amd import kernels
     return kernels
@@ -432,6 +437,29 @@ def test_randomised_configurations_match_oracle():
                 info = T.momentum_step_ref(c.states[0], c.p, g, c.ecc, **kw)
             c.compare(f"{what} step={step}", info, exact=kind != "adam" or dtype == torch.float32)
             c.resync_oracle()
+
+
+def test_step_kernels_are_resident_as_planned():
+    """Every step kernel bounds the workgroups resident on a compute unit by requesting unused LDS (streaming from
+    HBM degrades with too many bytes in flight per compute unit).  The request is derived from the device's LDS
+    size; the runtime's occupancy query must confirm the intended residency for every kernel family, in both grid
+    shapes."""
+    import ctypes
+
+    lib = _native_lib()
+    want_adam = {(0, 0): 23, (1, 0): 19, (1, 1): 19, (1, 2): 17, (2, 0): 19, (2, 1): 19, (2, 2): 17}
+    for (dtype, ecc), want in want_adam.items():
+        for quantized in (1, 0):
+            for multi in (0, 1):
+                t, a, lds = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+                rc = lib.fo_adam_step_residency(dtype, ecc, quantized, 1, multi, ctypes.byref(t), ctypes.byref(a), ctypes.byref(lds))
+                assert rc == 0 and t.value == want and a.value == want, (dtype, ecc, quantized, multi, t.value, a.value, lds.value)
+    for kind in (0, 1, 2):
+        for (dtype, ecc) in want_adam:
+            for multi in (0, 1):
+                t, a, lds = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+                rc = lib.fo_momentum_step_residency(dtype, ecc, 1, kind, multi, ctypes.byref(t), ctypes.byref(a), ctypes.byref(lds))
+                assert rc == 0 and t.value == 24 and a.value == 24, (kind, dtype, ecc, multi, t.value, a.value, lds.value)
 
 
 def test_the_binding_shown_in_the_integration_notes_runs():

@@ -1130,6 +1130,66 @@ def test_clearing_the_optimizer_state_restarts_the_moments():
         assert float(oa.state[a]["step"]) == 2.0
 
 
+def test_a_replaced_step_counter_object_is_honoured_by_the_cached_plan():
+    """Replacing a counter OBJECT (state[p]["step"] = torch.tensor(0.), as a hand-copied per-parameter state does)
+    leaves the pooled counters of the cached plan behind: the next step must notice, take the step number from the
+    new tensor, keep incrementing it, and save it in state_dict()."""
+    fo = _fo()
+    shapes = [5000, 4096, 70001]
+    pa, pb = _make_params(shapes, torch.bfloat16, 81), _make_params(shapes, torch.bfloat16, 81)
+    oa, ob = fo.FlashAdamW(pa, lr=1e-3), fo.FlashAdamW(pb, lr=1e-3)
+    for it in range(6):
+        _set_grads(pa, 810 + it)
+        _set_grads(pb, 810 + it)
+        if it == 3:
+            oa.state[pa[2]]["step"] = torch.tensor(0.0)
+            ob.state[pb[2]]["step"] = torch.tensor(0.0)
+        oa.step()
+        for p in pb:
+            ob.step_param(p)
+    for a, b in zip(pa, pb):
+        assert torch.equal(a, b)
+        sa, sb = _state_tensors(oa, a), _state_tensors(ob, b)
+        for k in sa:
+            assert parity.bits_equal(sa[k], sb[k]), k
+    assert [float(oa.state[p]["step"]) for p in pa] == [6.0, 6.0, 3.0]
+    assert [float(st["step"]) for st in oa.state_dict()["state"].values()] == [6.0, 6.0, 3.0]
+
+
+def test_a_moved_gradient_during_graph_capture_raises_before_any_launch():
+    """A cached multi-tensor plan whose gradient moved to another address needs its pointer table uploaded again.
+    Recorded into a HIP graph that copy would replay with whatever the staging buffer holds later, so step() must
+    raise on the host instead -- and stay usable afterwards."""
+    fo = _fo()
+    params = _make_params([5000, 33, 70001], torch.bfloat16, 82)
+    opt = fo.FlashLion(params, lr=1e-4)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for it in range(2):
+            _set_grads(params, 820 + it)
+            opt.step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    keep = [p.grad for p in params]                       # hold the old buffers so the new ones get new addresses
+    params[1].grad = torch.zeros_like(params[1])
+    assert params[1].grad.data_ptr() != keep[1].data_ptr()
+    before = [p.clone() for p in params]
+    graph = torch.cuda.CUDAGraph()
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")                   # torch remarks that the abandoned graph is empty
+        with pytest.raises(RuntimeError, match="cannot be recorded into a HIP graph"):
+            with torch.cuda.graph(graph):
+                opt.step()
+    torch.cuda.synchronize()
+    for p, b in zip(params, before):
+        assert torch.equal(p, b), "the refused step must not have launched anything"
+    _set_grads(params, 825)
+    opt.step()                                            # eager stepping still works and uploads the table
+    torch.cuda.synchronize()
+    assert not torch.equal(params[0], before[0])
+
+
 def test_rewritten_step_counters_are_honoured_by_the_cached_plan():
     """The per-parameter `step` scalars are ordinary state: zeroing them (a warm restart of the bias correction)
     or setting one of them apart must steer the next cached step exactly as it steers per-tensor stepping."""
