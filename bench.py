@@ -25,7 +25,9 @@ Workloads (``--workload``):
 
 Reported: ``value`` = parameters updated per second; ``roofline`` = algorithmic HBM bytes of one step divided
 by the average duration of a step (one event pair on the launch stream around the K timed steps, divided by K),
-against the 8 TB/s peak;
+against the 8 TB/s peak (``frac``; ``frac_wall`` divides by the host's wall clock per step instead);
+``parity`` (FlashAdamW workloads) = the HIP step against the CPU oracle on 2^20 and 2^20 + 17 elements after the
+timed region: raw code mismatch rate per step and the share of master weights beyond one unit;
 ``cpu_baseline`` = the CPU oracle (oracle/torch_oracle.py, all host cores) on a bounded sample of the same
 distribution, a reported baseline only.
 """
@@ -158,11 +160,27 @@ def build_workload(name: str, device):
     if name in ("ragged-lion", "ragged-sgdw"):
         lens = ragged_lengths()
         torch.manual_seed(3)
-        params = []
-        student = torch.distributions.StudentT(torch.tensor(3.0, device=device))
+        # parameters and gradients are carved from two flat buffers at 512-byte aligned offsets (what torch's
+        # allocator does for tensors allocated one after the other) and drawn with a few large kernels, so that
+        # the set-up does not issue tens of thousands of tiny launches (a profiler collecting counters per launch
+        # crashed on them)
+        offsets, total_padded = [], 0
         for n in lens:
-            p = torch.nn.Parameter((torch.randn(n, device=device) * 0.02).to(torch.bfloat16))
-            p.grad = (student.sample((n,)) * 1e-3).to(torch.bfloat16)
+            offsets.append(total_padded)
+            total_padded += (n + 255) // 256 * 256
+        flat_p = torch.empty(total_padded, dtype=torch.bfloat16, device=device)
+        flat_g = torch.empty(total_padded, dtype=torch.bfloat16, device=device)
+        for o in range(0, total_padded, 1 << 27):
+            m = min(1 << 27, total_padded - o)
+            flat_p[o:o + m] = (torch.randn(m, device=device) * 0.02).to(torch.bfloat16)
+            # Student-t with 3 degrees of freedom composed from normal draws, z / sqrt((z1^2 + z2^2 + z3^2) / 3)
+            z = torch.randn(4, m, device=device)
+            flat_g[o:o + m] = (z[0] / ((z[1] * z[1] + z[2] * z[2] + z[3] * z[3]) / 3.0).sqrt() * 1e-3).to(torch.bfloat16)
+            del z
+        params = []
+        for n, o in zip(lens, offsets):
+            p = torch.nn.Parameter(flat_p[o:o + n])
+            p.grad = flat_g[o:o + n]
             params.append(p)
         if name == "ragged-lion":
             opt = fo.FlashLion(params, lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1, master_weight_bits=24)
@@ -249,14 +267,51 @@ def cpu_baseline(steps: int = 5, warmup: int = 3, n: int = 1 << 26):
     }
 
 
+TRAFFIC_FILE = os.path.join("profiles", "hbm_traffic.json")
+
+
 def measured_traffic(workload: str):
-    """HBM bytes per step measured with rocprofv3 FETCH_SIZE / WRITE_SIZE (see profiles/), if recorded."""
-    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    """HBM bytes per step as recorded earlier with rocprofv3 FETCH_SIZE / WRITE_SIZE (profiles/hbm_traffic.json);
+    None when this workload has no entry.  This run does not measure it."""
     try:
-        with open(path) as f:
+        with open(os.path.join(ROOT, TRAFFIC_FILE)) as f:
             return json.load(f).get(workload, {}).get("bytes_per_step")
     except (OSError, ValueError):
         return None
+
+
+def parity_subcheck(device, ecc_dtype=torch.int8, steps: int = 4):
+    """HIP step against the CPU oracle on 2^20 and 2^20 + 17 bf16 elements (parameters N(0, 0.02), gradients
+    N(0, 1e-3) redrawn per step, FlashAdamW hyper-parameters of the throughput run), outside the timed region.
+    Reports the raw share of moment codes that differ (never by more than one step) per step, the first included,
+    and the share of master weights more than one unit of master precision away with no allowance."""
+    from flashoptim_amd import kernels as k
+    from oracle import torch_oracle as T
+    from tests import parity
+
+    out = {"sizes": [], "code_mismatch_fraction_per_step": [], "master_beyond_one_unit_per_step": []}
+    for n in (1 << 20, (1 << 20) + 17):
+        p = (torch.randn(n, generator=torch.Generator().manual_seed(0)) * 0.02).to(torch.bfloat16)
+        ecc = torch.zeros(n, dtype=ecc_dtype)
+        m, v = T.MomentState.zeros(n, True, True, torch.bfloat16), T.MomentState.zeros(n, False, True, torch.bfloat16)
+        gp, gecc = p.to(device), ecc.to(device)
+        gm, gms, gv, gvs = m.codes.to(device), m.scales.to(device), v.codes.to(device), v.scales.to(device)
+        rates, beyond = [], []
+        for step in range(1, steps + 1):
+            g = (torch.randn(n, generator=torch.Generator().manual_seed(1000 + step)) * 1e-3).to(torch.bfloat16)
+            k._fused_adam_step(gm, gms, gv, gvs, gp, g.to(device), gecc, 1e-3, 0.9, 0.999, 1e-8, 0.01 * 1e-3, True, step)
+            info = T.adam_step_ref(m, v, p, g, ecc, 1e-3, 0.9, 0.999, 1e-8, 0.01 * 1e-3, True, step)
+            rates.append(max(parity.check_codes(gm, m.codes, "bench m"), parity.check_codes(gv, v.codes, "bench v")))
+            parity.check_scales(gms, m.scales, "bench m scales")
+            parity.check_scales(gvs, v.scales, "bench v scales")
+            beyond.append(parity.check_master(gp, gecc, p, ecc, "bench master", step_size=info["update_scale"])[1])
+            for dst, src in ((p, gp), (ecc, gecc), (m.codes, gm), (m.scales, gms), (v.codes, gv), (v.scales, gvs)):
+                dst.copy_(src.cpu())  # the next comparison starts from identical inputs
+        out["sizes"].append(n)
+        out["code_mismatch_fraction_per_step"].append(rates)
+        out["master_beyond_one_unit_per_step"].append(beyond)
+    out["first_step_codes_identical"] = all(r[0] == 0.0 for r in out["code_mismatch_fraction_per_step"])
+    return out
 
 
 def main() -> None:
@@ -266,6 +321,7 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="llama8b-mwb24")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true", help="skip the HIP-vs-oracle sub-check that runs after the timed region")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the optimizer step is shard-local and this build has no "
@@ -328,16 +384,22 @@ def main() -> None:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "f32",  # the arithmetic type of the path; parameters and gradients are config.param_dtype
         "data": "synthetic",
         "config": {
             "workload": args.workload, "description": work["desc"], "optimizer": work["optimizer"],
+            "param_dtype": str(work["params"][0].dtype).replace("torch.", "").replace("bfloat16", "bf16").replace("float32", "f32"),
             "master_weight_bits": work["mwb"], "n_tensors": len(work["params"]), "n_params": total,
             "launch": work["launch"], "algorithmic_bytes_per_param": work["bpp"],
         },
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(args.workload),
+            "frac": achieved / HBM_PEAK_GBPS,
+            # the same algorithmic bytes over the host's wall clock per step (includes the host lead-in of the first step)
+            "frac_wall": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "traffic": measured_traffic(args.workload),
+            "traffic_source": TRAFFIC_FILE + " (rocprofv3 FETCH_SIZE + WRITE_SIZE, recorded earlier; not measured by this run)"
+                              if measured_traffic(args.workload) is not None else None,
             "step_device_ms_avg": avg_device_ms, "step_device_ms_avg_with_lead_in": first.elapsed_time(last) / args.steps,
             "step_device_ms_median": per_step[len(per_step) // 2], "step_device_ms_min": per_step[0],
             "algorithmic_bytes_per_step": step_bytes,
@@ -346,8 +408,11 @@ def main() -> None:
     if work.get("checkpoint_roundtrip"):
         out["config"]["checkpoint_roundtrip_bit_exact"] = checkpoint_roundtrip(work, device)
         out["config"]["checkpoint_bytes"] = work["checkpoint_bytes"]
+    adam_on_bf16 = work["optimizer"] == "FlashAdamW" and work["mwb"] in (24, 32)
+    del work
+    if adam_on_bf16 and not args.no_parity:
+        out["parity"] = parity_subcheck(device, torch.int8 if out["config"]["master_weight_bits"] == 24 else torch.int16)
     if not args.no_cpu_baseline:
-        del work
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
 

@@ -328,26 +328,17 @@ template <int DT> __device__ const StepTables<DT> kStepTables = StepTables<DT>()
 
 // The tables live in LDS during a kernel (1 KiB each, no replication: a few conflicted reads cost less than
 // filling a bank-replicated copy, because every short-lived workgroup fills its own).  A workgroup is one
-// wavefront; each lane copies four entries of each table with one 128-bit load (from L2) and one ds_write_b128.
-// Filling is split so that the global read is in flight together with the workgroup's streaming loads: fetch()
-// first, commit() just before the first lookup.  TABLES: 1 = first-moment codes, 2 = also the int8 ECC fractions.
+// wavefront; it fills each table with one 128-bit load per lane that writes straight into LDS (lane l delivers
+// entries 4l .. 4l+3; no registers, no ds_write).  The loads are issued before the workgroup's streaming loads and
+// the first lookup only waits for them, not for the streams issued after them.
+// TABLES: 1 = first-moment codes, 2 = also the int8 ECC fractions.
 template <int TABLES> struct StepLut {
     static constexpr int kFloats = TABLES > 0 ? 256 * TABLES : 4;
-    struct Frag { float v[TABLES > 0 ? 4 * TABLES : 1]; };
-    __device__ __forceinline__ static Frag fetch(const float* table) {
-        Frag f;
+    __device__ __forceinline__ static void fill(float* lut, const float* table) {
 #pragma unroll
         for (int t = 0; t < TABLES; ++t)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) f.v[4 * t + j] = ((const FO_GLOBAL float*)table)[256 * t + (threadIdx.x & 63) * 4 + j];
-        return f;
-    }
-    __device__ __forceinline__ static void commit(float* lut, const Frag& f) {
-#pragma unroll
-        for (int t = 0; t < TABLES; ++t)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) lut[256 * t + (threadIdx.x & 63) * 4 + j] = f.v[4 * t + j];
-        __syncthreads();  // a single-wavefront workgroup needs no hardware barrier; the compiler drops it
+            __builtin_amdgcn_global_load_lds((const FO_GLOBAL void*)(table + 256 * t + (threadIdx.x & 63) * 4),
+                                             (__attribute__((address_space(3))) void*)(lut + 256 * t), 16, 0, 0);
     }
 };
 __device__ __forceinline__ float lookup_mom(const float* lut, u32 byte) { return lut[byte]; }

@@ -159,48 +159,33 @@ template <class Op> struct Span {
 // four consecutive spans removes that over-fetch exactly but streams 5 % slower (4 KiB per XCD instead of
 // 1 KiB), so the identity order stays.
 
-// One span starting at element `base` of tensor t.  All loads are issued first, `between()` runs while they are
-// in flight (the workgroup commits the LDS table there), then the span is finished.
-template <class Op, class Between>
+// One span starting at element `base` of tensor t: all loads are issued first, then the span is finished.
+template <class Op>
 __device__ __forceinline__ void run_span(const TensorPtrs& t, int64_t base, bool aligned, const typename Op::Hyper& h,
-                                         const float* lut, Between&& between) {
+                                         const float* lut) {
     const Where first{base, (int)(threadIdx.x & 63) * Op::kEpl};
     typename Op::Raw raw;
     // workgroup-uniform choice of the access mode
     if (aligned) {
         if (base + Span<Op>::kElems <= t.n) {
             Op::template load<kVector>(t, first, raw);
-            between();
             Op::template finish<kVector>(t, first, raw, h, lut);
         } else {
             Op::template load<kLane>(t, first, raw);
-            between();
             Op::template finish<kLane>(t, first, raw, h, lut);
         }
     } else {
-        between();
         Op::template load<kGuarded>(t, first, raw);
         Op::template finish<kGuarded>(t, first, raw, h, lut);
     }
 }
 
-// Commits the code tables to LDS once per workgroup, at the first call.
-template <int TABLES> struct LutCommit {
-    float* lut; typename StepLut<TABLES>::Frag frag; bool done;
-    __device__ __forceinline__ void operator()() {
-        if constexpr (TABLES > 0) {
-            if (!done) { StepLut<TABLES>::commit(lut, frag); done = true; }
-        }
-    }
-};
-
 template <class Op>
 __global__ __launch_bounds__(kBlockThreads) void step_single_kernel(TensorPtrs t, typename Op::Hyper h) {
     __shared__ __align__(16) float lut[StepLut<Op::kLutTables>::kFloats];
     const int64_t base = (int64_t)blockIdx.x * Span<Op>::kElems;
-    LutCommit<Op::kLutTables> commit{lut, {}, false};
-    if constexpr (Op::kLutTables > 0) commit.frag = StepLut<Op::kLutTables>::fetch(kStepTables<Op::kDtype>.v);
-    run_span<Op>(t, base, all_aligned16(t), h, lut, commit);
+    if constexpr (Op::kLutTables > 0) StepLut<Op::kLutTables>::fill(lut, kStepTables<Op::kDtype>.v);
+    run_span<Op>(t, base, all_aligned16(t), h, lut);
 }
 
 // Workgroup b works on chunk b / kPerTile and takes span b % kPerTile of each of the chunk's tiles.
@@ -212,13 +197,12 @@ __global__ __launch_bounds__(kBlockThreads) void step_multi_kernel(const fo_tens
     const unsigned b = blockIdx.x;
     const fo_chunk ck = chunks[b / kPerTile];
     const TensorPtrs t = load_desc(descs + ck.tensor);
-    LutCommit<Op::kLutTables> commit{lut, {}, false};
-    if constexpr (Op::kLutTables > 0) commit.frag = StepLut<Op::kLutTables>::fetch(kStepTables<Op::kDtype>.v);
+    if constexpr (Op::kLutTables > 0) StepLut<Op::kLutTables>::fill(lut, kStepTables<Op::kDtype>.v);
     const bool aligned = all_aligned16(t);
     const int64_t in_tile = (int64_t)(b % kPerTile) * Span<Op>::kElems;
     for (int i = 0; i < ck.n_tiles; ++i) {
         const int64_t base = ((int64_t)ck.first_tile + i) * kTileElems + in_tile;
-        if (base < t.n) run_span<Op>(t, base, aligned, h, lut, commit);
+        if (base < t.n) run_span<Op>(t, base, aligned, h, lut);
     }
 }
 

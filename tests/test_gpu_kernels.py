@@ -447,7 +447,7 @@ def test_step_kernels_are_resident_as_planned():
     import ctypes
 
     lib = _native_lib()
-    want_adam = {(0, 0): 23, (1, 0): 19, (1, 1): 19, (1, 2): 17, (2, 0): 19, (2, 1): 19, (2, 2): 17}
+    want_adam = {(0, 0): 23, (1, 0): 20, (1, 1): 20, (1, 2): 19, (2, 0): 20, (2, 1): 20, (2, 2): 19}
     for (dtype, ecc), want in want_adam.items():
         for quantized in (1, 0):
             for multi in (0, 1):
@@ -459,7 +459,7 @@ def test_step_kernels_are_resident_as_planned():
             for multi in (0, 1):
                 t, a, lds = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
                 rc = lib.fo_momentum_step_residency(dtype, ecc, 1, kind, multi, ctypes.byref(t), ctypes.byref(a), ctypes.byref(lds))
-                assert rc == 0 and t.value == 24 and a.value == 24, (kind, dtype, ecc, multi, t.value, a.value, lds.value)
+                assert rc == 0 and t.value == 26 and a.value == 26, (kind, dtype, ecc, multi, t.value, a.value, lds.value)
 
 
 def test_the_binding_shown_in_the_integration_notes_runs():
