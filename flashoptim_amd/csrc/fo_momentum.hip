@@ -85,7 +85,8 @@ template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumOp {
     using Hyper = MomentumHyper;
     static constexpr int kLutTables = ECCB == 1 ? 2 : ((QUANT && KIND != KIND_PLAIN) ? 1 : 0);  // LDS code tables (fo_device.h)
     static constexpr int kDtype = DT;
-    static constexpr int kWorkgroupsPerCu = 26;  // measured on MI355X: 24 best for the 8B list, 27-30 for 4096 ragged tensors (3 KiB of loads per wavefront)
+    // measured on MI355X: 24 best for the 8B list, 27-30 for 4096 ragged tensors (3 KiB of loads per wavefront)
+    static constexpr int kWorkgroupsPerCu = 26;
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = MomentumRaw<DT, ECCB, QUANT, KIND>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {
