@@ -268,10 +268,7 @@ inline AdamHyper make_adam_hyper(float lr, float beta1, float beta2, float eps, 
 // Which variants follow the reference's update operation by operation (EXACT) instead of the folded form:
 // fp32 parameters, where one fp32 ulp is the master precision and the 16.25 bytes per element leave room
 // for the extra arithmetic.  Narrow parameters use the folded update (see adam_apply).
-#ifndef FO_EXACT_RULE
-#define FO_EXACT_RULE (DT == DT_F32)
-#endif
-template <int DT, int ECCB> struct AdamExact { static constexpr bool value = FO_EXACT_RULE; };
+template <int DT, int ECCB> struct AdamExact { static constexpr bool value = DT == DT_F32; };
 
 // New moments from the dequantised pieces.
 //   EXACT = false: the EMA decay is folded into the group scale (one multiply per lane instead of one per
