@@ -43,6 +43,7 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
     constexpr int PB = DTypeInfo<DT>::bytes;
     constexpr int SB = QUANT ? 1 : PB;
     constexpr bool EXACT = AdamExact<DT, ECCB>::value;
+    constexpr bool MAY_BE_QUICK = QUANT && AdamQuickRequant<DT, ECCB>::value;  // fo_math.h: "two requantisers"
     const int64_t n = t.n;
     const bool live_group = FAST == kVector || w.first() < n;  // the lane owns at least one real element
     const float sm = f16_bits_to_f32(raw.sm), sv = f16_bits_to_f32(raw.sv);
@@ -64,9 +65,9 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
         }
         float pk = p[k];
         if constexpr (DECOUPLED) pk = pk * h.one_m_wd;                              // ref:2363-2364
-        // sqrt(v), correctly rounded: the requantiser needs exactly this value (ref:2393) and the folded update
-        // shares it
-        const float rk = (QUANT || !EXACT) ? sqrt_corrected(vn) : 0.0f;
+        // sqrt(v): the requantiser needs it (ref:2393) and the folded update shares it.  The folded update is content
+        // with the instruction's value; the exact requantiser replaces it by the correctly rounded one below.
+        const float rk = (QUANT || !EXACT) ? (MAY_BE_QUICK ? hw::sqrt(vn) : sqrt_corrected(vn)) : 0.0f;
         p[k] = adam_apply<EXACT>(pk, mn, vn, rk, h);                                // ref:2368-2375
         m[k] = mn; r[k] = rk; v[k] = vn;
     }
@@ -77,6 +78,15 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
     store_lane<ECCB, EPL, FAST>(eout, t.ecc, w, n);
 
     if constexpr (QUANT) {
+        // wavefront-uniform: one group of the span that starts from a zero state sends the whole span through the
+        // exact requantiser
+        const bool quick = MAY_BE_QUICK && __builtin_amdgcn_ballot_w64(scale_is_zero(raw.sm) || scale_is_zero(raw.sv)) == 0;
+        if constexpr (MAY_BE_QUICK) {
+            if (!quick) {
+#pragma unroll
+                for (int k = 0; k < EPL; ++k) r[k] = sqrt_corrected(v[k]);
+            }
+        }
         float am = 0.0f, av = 0.0f;
 #pragma unroll
         for (int k = 0; k < EPL; k += 2) {  // pairs, so that each step is one three-operand max
@@ -86,7 +96,16 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
         // group absmax (ref:2399-2404)
         am = fmaxf(group_max<EPL>(am), 1e-12f);
         av = fmaxf(group_max<EPL>(av), 1e-12f);
-        if constexpr (EPL == 8) {
+        if constexpr (MAY_BE_QUICK) {
+            static_assert(EPL == 8, "2-byte parameters");
+            if (quick) {
+                quantize_mom<EPL, true>(m, am, raw.m);
+                quantize_var<EPL, true>(r, av, raw.v);
+            } else {
+                quantize_mom<EPL, false>(m, am, raw.m);
+                quantize_var<EPL, false>(r, av, raw.v);
+            }
+        } else if constexpr (EPL == 8) {
             quantize_mom<EPL>(m, am, raw.m);
             quantize_var<EPL>(r, av, raw.v);
         } else {

@@ -64,6 +64,7 @@ static inline float nudge(float exact, float x) {
 }
 static inline float rcp(float x) { return nudge((float)(1.0 / (double)x), x); }
 static inline float rsq(float x) { return nudge((float)(1.0 / sqrt((double)x)), x); }
+static inline float sqrt(float x) { return nudge(sqrtf(x), x); }
 static inline float ldexp(float x, int e) { return ldexpf(x, e); }
 static inline float med3(float x, float lo, float hi) { return fminf(fmaxf(x, lo), hi); }
 static inline int floor_to_int(float x) { return (int)floorf(x); }
@@ -71,6 +72,7 @@ static inline float fma(float a, float b, float c) { return __builtin_fmaf(a, b,
 #else
 FO_FN float rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 FO_FN float rsq(float x) { return __builtin_amdgcn_rsqf(x); }
+FO_FN float sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
 FO_FN float ldexp(float x, int e) { return __builtin_amdgcn_ldexpf(x, e); }
 FO_FN float med3(float x, float lo, float hi) { return __builtin_amdgcn_fmed3f(x, lo, hi); }
 // (int)floor(x) in one instruction
@@ -220,6 +222,27 @@ FO_FN float quantize_var_rounded(float r, float av, float rav) {
     const float q = div_corrected(r, av, rav);
     return q * 255.0f + 0.5f;  // non-negative: truncation is the floor
 }
+// Two requantisers.  The exact one above costs two corrected quotients per first-moment value and a corrected
+// quotient plus a corrected square root per second-moment value.  What it buys shows where the pre-rounding value
+// of a code lies on a rounding boundary k + 1/2 to the last bit, and that happens in bulk only when the new
+// moments are a narrow-precision gradient times a constant, i.e. when the old state of the group is zero (first
+// step, or a group whose gradients have been zero so far): 0.3 % of the second-moment values of such a group sit
+// exactly on a boundary, and which side they fall on depends on every rounding of the reference's formula.  Once
+// the old state contributes, the values are generic and a formula that is a few ulps off picks another code only
+// for the 1e-5 of the elements whose value lies within those ulps of a boundary.
+// The quick forms are the same real-number formulas with the quotients merged and approximate (a few ulps), the
+// rounding still floor(x + 0.5).  Adam on 2-byte parameters with no or a 1-byte ECC (AdamQuickRequant; its update
+// is folded and therefore already agrees with the reference to rounding error only, see adam_apply) uses them for
+// every wavefront span in which no group starts from a zero state (scale_is_zero); a span with such a group, and
+// every other kernel, uses the exact forms.  rav255 = 255 * rcp(group maximum of sqrt(v)); the quick path takes
+// sqrt(v) from hw::sqrt.
+FO_FN float quantize_mom_quick(float m, float am) {
+    const float t = m * hw::rcp(am + fabsf(m));  // = nm / (1 + |nm|), nm = m / am
+    return hw::fma(t, 254.0f, 0.5f);
+}
+FO_FN float quantize_var_quick(float r, float rav255) { return hw::fma(r, rav255, 0.5f); }
+// A stored fp16 group scale of zero: every element of the group is zero (ref:2399-2404 store the absmax).
+FO_FN bool scale_is_zero(uint16_t f16_bits) { return (f16_bits & 0x7fffu) == 0; }
 FO_FN u32 quantize_mom_code(float m, float am, float ram) { return (u32)hw::floor_to_int(quantize_mom_rounded(m, am, ram)); }
 FO_FN u32 quantize_var_code(float r, float av, float rav) { return (u32)(int)quantize_var_rounded(r, av, rav); }
 
@@ -269,6 +292,9 @@ inline AdamHyper make_adam_hyper(float lr, float beta1, float beta2, float eps, 
 // fp32 parameters, where one fp32 ulp is the master precision and the 16.25 bytes per element leave room
 // for the extra arithmetic.  Narrow parameters use the folded update (see adam_apply).
 template <int DT, int ECCB> struct AdamExact { static constexpr bool value = DT == DT_F32; };
+// Variants whose wavefronts may take the quick requantiser: those with the folded update, except the ones with a
+// 2-byte ECC, whose 14.25 bytes per element hide the exact requantiser's arithmetic (measured: no gain).
+template <int DT, int ECCB> struct AdamQuickRequant { static constexpr bool value = !AdamExact<DT, ECCB>::value && ECCB != 2; };
 
 // New moments from the dequantised pieces.
 //   EXACT = false: the EMA decay is folded into the group scale (one multiply per lane instead of one per

@@ -87,27 +87,27 @@ __device__ __forceinline__ void write_master(const float (&p)[EPL], Pack<DTypeIn
 // Quantises the lane's first-moment values against the group absmax `am` (shared by the group's lanes, clamped
 // at 1e-12) and the lane's sqrt(v) values against the group maximum `av`; the rounding is the reference's
 // (fo_math.h: quantize_mom_rounded, quantize_var_rounded; ref:2405-2419, 1703-1710).
-template <int EPL>
+template <int EPL, bool QUICK = false>
 __device__ __forceinline__ void quantize_mom(const float (&m)[EPL], float am, Pack<1, EPL>& out) {
     static_assert(EPL == 8, "two dwords of codes per lane");
-    const float ram = hw::rcp(am);
+    const float ram = QUICK ? 0.0f : hw::rcp(am);
     float lo[4], hi[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        lo[k] = quantize_mom_rounded(m[k], am, ram);
-        hi[k] = quantize_mom_rounded(m[k + 4], am, ram);
+        lo[k] = QUICK ? quantize_mom_quick(m[k], am) : quantize_mom_rounded(m[k], am, ram);
+        hi[k] = QUICK ? quantize_mom_quick(m[k + 4], am) : quantize_mom_rounded(m[k + 4], am, ram);
     }
     convert_pack8<kFloor, kFloor>(lo, hi, out.w[0], out.w[1]);
 }
-template <int EPL>
+template <int EPL, bool QUICK = false>
 __device__ __forceinline__ void quantize_var(const float (&r)[EPL], float av, Pack<1, EPL>& out) {
     static_assert(EPL == 8, "two dwords of codes per lane");
-    const float rav = hw::rcp(av);
+    const float rav = QUICK ? hw::rcp(av) * 255.0f : hw::rcp(av);
     float lo[4], hi[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        lo[k] = quantize_var_rounded(r[k], av, rav);
-        hi[k] = quantize_var_rounded(r[k + 4], av, rav);
+        lo[k] = QUICK ? quantize_var_quick(r[k], rav) : quantize_var_rounded(r[k], av, rav);
+        hi[k] = QUICK ? quantize_var_quick(r[k + 4], rav) : quantize_var_rounded(r[k + 4], av, rav);
     }
     convert_pack8<kTrunc, kTrunc>(lo, hi, out.w[0], out.w[1]);
 }

@@ -229,6 +229,35 @@ def test_adam_headline_config_code_mismatch_rate(ecc_dtype):
         assert max(a for a, _ in stats) < parity.CODE_MISMATCH_FRACTION
 
 
+@pytest.mark.parametrize("dtype,ecc_dtype", [(torch.bfloat16, torch.int8), (torch.float16, torch.int8), (torch.bfloat16, None), (torch.bfloat16, torch.int16)])
+def test_adam_groups_that_start_from_zero_get_the_exact_requantiser(dtype, ecc_dtype):
+    """Two steps, then 2 % of the groups are reset to a zero state (as if they had seen no gradient yet) and a
+    third step is taken: every code of a reset group equals the oracle's, whichever requantiser the rest of its
+    wavefront span would have taken; all other codes meet the usual rate."""
+    k = _k()
+    n = (1 << 17) + 17
+    c = _Case(n, dtype, ecc_dtype, True, 2, seed=5)
+    lr, b1, b2, eps, wd = 1e-3, 0.9, 0.999, 1e-8, 1e-5
+    for step in (1, 2):
+        g = _rand(n, 1e-3, 50 + step).to(dtype)
+        (m, ms), (v, vs) = c.gstates
+        k._fused_adam_step(m, ms, v, vs, c.gp, g.to(DEV), c.gecc, lr, b1, b2, eps, wd, True, step, quantize_optim_states=True)
+    n_groups = (n + 31) // 32
+    reset = torch.rand(n_groups, generator=torch.Generator().manual_seed(9)) < 0.02
+    in_reset = reset.repeat_interleave(32)[:n]
+    for codes, scales in c.gstates:
+        codes[in_reset.to(DEV)] = 0
+        scales[reset.to(DEV)] = 0
+    c.resync_oracle()
+    g = _rand(n, 1e-3, 77).to(dtype)
+    (m, ms), (v, vs) = c.gstates
+    k._fused_adam_step(m, ms, v, vs, c.gp, g.to(DEV), c.gecc, lr, b1, b2, eps, wd, True, 3, quantize_optim_states=True)
+    info = T.adam_step_ref(c.states[0], c.states[1], c.p, g, c.ecc, lr, b1, b2, eps, wd, True, 3)
+    c.compare(f"adam {dtype} ecc={ecc_dtype} after a partial reset", info, exact=False)
+    for s, (a, _) in zip(c.states, c.gstates):
+        assert torch.equal(a.cpu()[in_reset], s.codes[in_reset]), "a group that started from zero differs from the oracle"
+
+
 def test_adam_unaligned_pointers():
     _adam_steps(5000, torch.bfloat16, torch.int8, True, True, steps=3, seed=9, offset=3)
     _adam_steps(5000, torch.float32, None, True, True, steps=3, seed=9, offset=1)
