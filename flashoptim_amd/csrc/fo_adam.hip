@@ -129,10 +129,11 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED> struct AdamOp {
     using Hyper = AdamHyper;
     static constexpr int kLutTables = ECCB == 1 ? 2 : (QUANT ? 1 : 0);  // LDS code tables (fo_device.h)
     static constexpr int kDtype = DT;
-    // measured on MI355X with the 8B-parameter step (plateaus three to four wide): 19-22 resident workgroups per
-    // compute unit for 2-byte parameters with no or a 1-byte ECC (3.6-4.1 KiB of loads per wavefront), 19 with a
-    // 2-byte ECC (4.6 KiB), 23 for fp32 parameters (2.5 KiB)
-    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 23 : (ECCB == 2 ? 19 : 20);
+    // measured on MI355X with the 8B-parameter step and this file's ILP-oriented instruction schedule: 14-15
+    // resident workgroups per compute unit for 2-byte parameters with no or a 1-byte ECC (3.6-4.1 KiB of loads per
+    // wavefront; 13 and 16 are two to four points worse), 16 with a 2-byte ECC (4.6 KiB), 18-20 for fp32 parameters
+    // (2.5 KiB)
+    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 20 : (ECCB == 2 ? 16 : 15);
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {

@@ -476,7 +476,7 @@ def test_step_kernels_are_resident_as_planned():
     import ctypes
 
     lib = _native_lib()
-    want_adam = {(0, 0): 23, (1, 0): 20, (1, 1): 20, (1, 2): 19, (2, 0): 20, (2, 1): 20, (2, 2): 19}
+    want_adam = {(0, 0): 20, (1, 0): 15, (1, 1): 15, (1, 2): 16, (2, 0): 15, (2, 1): 15, (2, 2): 16}
     for (dtype, ecc), want in want_adam.items():
         for quantized in (1, 0):
             for multi in (0, 1):
