@@ -85,7 +85,9 @@ template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumOp {
     using Hyper = MomentumHyper;
     static constexpr int kLutTables = ECCB == 1 ? 2 : ((QUANT && KIND != KIND_PLAIN) ? 1 : 0);  // LDS code tables (fo_device.h)
     static constexpr int kDtype = DT;
-    // measured on MI355X: 24 best for the 8B list, 27-30 for 4096 ragged tensors (3 KiB of loads per wavefront)
+    // measured on MI355X (3 KiB of loads per wavefront): 24 best for the 8B list, 26-30 for 4096 ragged tensors.
+    // (The ILP-oriented schedule that fo_adam.hip is built with gains 1-2 points on the 8B list at 18-20 resident
+    // workgroups and loses as much on the ragged list, which wants more than the 24 that its 80 VGPRs allow.)
     static constexpr int kWorkgroupsPerCu = 26;
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = MomentumRaw<DT, ECCB, QUANT, KIND>;
