@@ -180,9 +180,8 @@ __device__ __forceinline__ void run_span(const TensorPtrs& t, int64_t base, bool
     }
 }
 
-// The second launch bound (wavefronts per SIMD) keeps the register count within what the planned residency needs.
 template <class Op>
-__global__ __launch_bounds__(kBlockThreads, (Op::kWorkgroupsPerCu + 3) / 4) void step_single_kernel(TensorPtrs t, typename Op::Hyper h) {
+__global__ __launch_bounds__(kBlockThreads) void step_single_kernel(TensorPtrs t, typename Op::Hyper h) {
     __shared__ __align__(16) float lut[StepLut<Op::kLutTables>::kFloats];
     const int64_t base = (int64_t)blockIdx.x * Span<Op>::kElems;
     if constexpr (Op::kLutTables > 0) StepLut<Op::kLutTables>::fill(lut, kStepTables<Op::kDtype>.v);
@@ -191,7 +190,7 @@ __global__ __launch_bounds__(kBlockThreads, (Op::kWorkgroupsPerCu + 3) / 4) void
 
 // Workgroup b works on chunk b / kPerTile and takes span b % kPerTile of each of the chunk's tiles.
 template <class Op>
-__global__ __launch_bounds__(kBlockThreads, (Op::kWorkgroupsPerCu + 3) / 4) void step_multi_kernel(const fo_tensor_desc* __restrict__ descs,
+__global__ __launch_bounds__(kBlockThreads) void step_multi_kernel(const fo_tensor_desc* __restrict__ descs,
                                                                    const fo_chunk* __restrict__ chunks, typename Op::Hyper h) {
     __shared__ __align__(16) float lut[StepLut<Op::kLutTables>::kFloats];
     constexpr int kPerTile = Span<Op>::kPerTile;
