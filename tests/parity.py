@@ -4,10 +4,12 @@ What the kernels promise (flashoptim_amd/csrc/fo_math.h) and what the tests ther
 identical inputs:
 * SGD / SGDW / Nesterov / Lion steps, the momentum-free SGD step, Adam with fp32 parameters, unquantised states, the
   standalone codec and the standalone ECC kernels: every output bit equals the oracle's (`bits_equal`);
-* Adam with bf16 / fp16 parameters (folded update): the requantiser itself is exact, but the new moments come out
-  of fused multiply-adds and may differ from the oracle's by an ulp, so
+* Adam with bf16 / fp16 parameters (folded update): the new moments come out of fused multiply-adds and may differ
+  from the oracle's by an ulp, and wavefront spans in which every group carries state requantise with the quick
+  forms (a few ulps off; no or 1-byte ECC only), so
   - 8-bit moment codes never differ by more than +-1 code step and differ on fewer than 0.01 % of the elements
-    (measured 1e-6 .. 1e-5; exactly 0 on a first step from zero states, where m and v are formed identically);
+    (measured 1e-6 .. 2.5e-5; exactly 0 on a first step from zero states and in any group that starts from zero,
+    where m and v are formed identically and the exact requantiser runs);
   - fp16 group scales: equal, or one fp16 ulp apart on fewer than 0.1 % of the groups;
   - master weights (narrow parameter + ECC): within one unit of master precision, i.e. half-ulp(narrow)/127 for
     24-bit, /32767 for 32-bit masters; plus one fp32 ulp (the updated value is rounded to fp32 before it is
