@@ -12,6 +12,9 @@ Workloads (``--workload``):
                   FlashAdamW, master_weight_bits=24, one multi-tensor launch per step: the configuration the
                   headline metric is quoted on.
   llama8b-mwb32   same shapes, master_weight_bits=32 (int16 correction term).
+  llama8b-mwb24-exact / llama8b-mwb32-exact
+                  the same with FlashAdamW(exact_update=True): the update evaluated operation by operation
+                  (bit-exact with the CPU oracle), to show what that costs.
   flat-2p30       one flat bf16 tensor of 2^30 elements, FlashAdamW, master_weight_bits=24.
   llama8b-lion / llama8b-sgdw
                   the same parameter list under FlashLion / FlashSGDW (one quantised moment), master_weight_bits=24.
@@ -126,17 +129,19 @@ def build_workload(name: str, device):
     import flashoptim_amd as fo
 
     hp = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
-    if name in ("llama8b-mwb24", "llama8b-mwb32"):
+    if name in ("llama8b-mwb24", "llama8b-mwb32", "llama8b-mwb24-exact", "llama8b-mwb32-exact"):
         shapes = llama3_8b_shapes()
         g = torch.Generator().manual_seed(2)
         scales = (10.0 ** (torch.rand(len(shapes), generator=g) * 2 - 1)).tolist()
         params = make_params(shapes, torch.bfloat16, device, scales)
-        mwb = 24 if name.endswith("24") else 32
-        opt = fo.FlashAdamW(params, master_weight_bits=mwb, **hp)
+        mwb = 24 if "mwb24" in name else 32
+        exact = name.endswith("-exact")
+        opt = fo.FlashAdamW(params, master_weight_bits=mwb, exact_update=exact, **hp)
         return dict(params=params, opt=opt, step=rotating_gradients(params, opt.step, device, scales),
                     bpp=bytes_per_param(2, 1 if mwb == 24 else 2, 2),
                     desc=f"Llama-3-8B-shaped parameter list, bf16, FlashAdamW, master_weight_bits={mwb}, "
-                         "gradients redrawn per step (3 rotating sets)",
+                         + ("exact_update=True (operation-by-operation update), " if exact else "")
+                         + "gradients redrawn per step (3 rotating sets)",
                     launch="one multi-tensor launch per step", optimizer="FlashAdamW", mwb=mwb)
     if name in ("llama8b-lion", "llama8b-sgdw"):
         shapes = llama3_8b_shapes()
@@ -280,7 +285,7 @@ def measured_traffic(workload: str):
         return None
 
 
-def parity_subcheck(device, ecc_dtype=torch.int8, steps: int = 4):
+def parity_subcheck(device, ecc_dtype=torch.int8, steps: int = 4, exact_update: bool = False):
     """HIP step against the CPU oracle on 2^20 and 2^20 + 17 bf16 elements (parameters N(0, 0.02), gradients
     N(0, 1e-3) redrawn per step, FlashAdamW hyper-parameters of the throughput run), outside the timed region.
     Reports the raw share of moment codes that differ (never by more than one step) per step, the first included,
@@ -299,7 +304,8 @@ def parity_subcheck(device, ecc_dtype=torch.int8, steps: int = 4):
         rates, beyond = [], []
         for step in range(1, steps + 1):
             g = (torch.randn(n, generator=torch.Generator().manual_seed(1000 + step)) * 1e-3).to(torch.bfloat16)
-            k._fused_adam_step(gm, gms, gv, gvs, gp, g.to(device), gecc, 1e-3, 0.9, 0.999, 1e-8, 0.01 * 1e-3, True, step)
+            k._fused_adam_step(gm, gms, gv, gvs, gp, g.to(device), gecc, 1e-3, 0.9, 0.999, 1e-8, 0.01 * 1e-3, True, step,
+                               exact_update=exact_update)
             info = T.adam_step_ref(m, v, p, g, ecc, 1e-3, 0.9, 0.999, 1e-8, 0.01 * 1e-3, True, step)
             rates.append(max(parity.check_codes(gm, m.codes, "bench m"), parity.check_codes(gv, v.codes, "bench v")))
             parity.check_scales(gms, m.scales, "bench m scales")
@@ -409,9 +415,11 @@ def main() -> None:
         out["config"]["checkpoint_roundtrip_bit_exact"] = checkpoint_roundtrip(work, device)
         out["config"]["checkpoint_bytes"] = work["checkpoint_bytes"]
     adam_on_bf16 = work["optimizer"] == "FlashAdamW" and work["mwb"] in (24, 32)
+    exact_update = args.workload.endswith("-exact")
     del work
     if adam_on_bf16 and not args.no_parity:
-        out["parity"] = parity_subcheck(device, torch.int8 if out["config"]["master_weight_bits"] == 24 else torch.int16)
+        out["parity"] = parity_subcheck(device, torch.int8 if out["config"]["master_weight_bits"] == 24 else torch.int16,
+                                        exact_update=exact_update)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

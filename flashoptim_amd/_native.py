@@ -61,11 +61,13 @@ SIGNATURES = {
     "fo_last_error": (ctypes.c_char_p, []),
     "fo_device_compute_units": (_i32, [_i32]),
     "fo_adam_step": (_i32, [_vp] * 7 + [_i64, _i32, _i32, _i32] + [_f32] * 5 + [_i32, _i32, _vp]),
+    "fo_adam_step_exact": (_i32, [_vp] * 7 + [_i64, _i32, _i32, _i32] + [_f32] * 5 + [_i32, _i32, _vp]),
     "fo_momentum_step": (_i32, [_vp] * 5 + [_i64, _i32, _i32, _i32] + [_f32] * 4 + [_i32, _i32, _i32, _vp]),
     "fo_sgd_plain_step": (_i32, [_vp] * 3 + [_i64, _i32, _i32, _f32, _f32, _i32, _vp]),
     "fo_count_chunks": (_i64, [_vp, _i64, _i32]),
     "fo_build_chunks": (_i64, [_vp, _i64, _i32, _vp, _i64]),
     "fo_multi_adam_step": (_i32, [_vp, _i64, _vp, _i64, _i32, _i32, _i32] + [_f32] * 5 + [_i32, _i32, _vp]),
+    "fo_multi_adam_step_exact": (_i32, [_vp, _i64, _vp, _i64, _i32, _i32, _i32] + [_f32] * 5 + [_i32, _i32, _vp]),
     "fo_multi_adam_step_static": (_i32, [_vp, _i64, _i32, _i32, _i32] + [_f32] * 5 + [_i32, _i32, _vp]),
     "fo_multi_momentum_step": (_i32, [_vp, _i64, _vp, _i64, _i32, _i32, _i32] + [_f32] * 4 + [_i32, _i32, _i32, _vp]),
     "fo_multi_sgd_plain_step": (_i32, [_vp, _i64, _vp, _i64, _i32, _i32, _f32, _f32, _i32, _vp]),

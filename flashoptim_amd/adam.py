@@ -2,6 +2,7 @@
 
 from __future__ import annotations
 
+import os
 from collections.abc import Iterable
 from typing import Any, Literal, Optional
 
@@ -21,6 +22,12 @@ class FlashAdam(FlashOptimizer):
         eps: added to the denominator (default 1e-8).
         weight_decay: L2 coefficient (default 0).
         quantize, compress_state_dict, master_weight_bits, check_numerics, fused: see :class:`FlashOptimizer`.
+        exact_update: keyword-only, not in the reference (default: the ``FLASHOPTIM_EXACT_ADAM`` environment variable,
+            else False).  Evaluate the update operation by operation as the reference writes it for bf16 / fp16
+            parameters too (fp32 parameters always are): master weights and state codes then equal an IEEE
+            evaluation of the reference's formulas bit for bit, at 10-20 % less throughput.  With False the bias
+            corrections and the learning rate are folded into two constants, which leaves 1e-4 (24-bit masters) to
+            2e-2 (32-bit masters) of the master weights more than one unit of master precision away.
     """
 
     def __init__(
@@ -35,6 +42,8 @@ class FlashAdam(FlashOptimizer):
         master_weight_bits: Literal[24, 32] | None = 24,
         check_numerics: bool = False,
         fused: bool = True,
+        *,
+        exact_update: Optional[bool] = None,
     ):
         if not 0.0 <= eps:
             raise ValueError(f"Invalid epsilon value: {eps}")
@@ -45,6 +54,9 @@ class FlashAdam(FlashOptimizer):
             raise ValueError(f"Invalid weight_decay value: {weight_decay}")
         self._decoupled = False
         self._decouple_lr = False
+        if exact_update is None:
+            exact_update = os.environ.get("FLASHOPTIM_EXACT_ADAM", "0").strip().lower() not in ("", "0", "false", "no")
+        self._exact_update = bool(exact_update)
         super().__init__(
             params=params, lr=lr, defaults={"betas": betas, "weight_decay": weight_decay, "eps": eps},
             quantize=quantize, compress_state_dict=compress_state_dict, master_weight_bits=master_weight_bits,
@@ -88,7 +100,7 @@ class FlashAdam(FlashOptimizer):
         if self._decoupled:  # the kernel multiplies the weights by 1 - weight_decay (ref:1894-1898)
             weight_decay *= (lr / hparams["initial_lr"]) if self._decouple_lr else lr
         return dict(lr=lr, beta1=hparams["betas"][0], beta2=hparams["betas"][1], eps=hparams["eps"],
-                    weight_decay=weight_decay, decoupled=self._decoupled, step=step)
+                    weight_decay=weight_decay, decoupled=self._decoupled, step=step, exact_update=self._exact_update)
 
 
 class FlashAdamW(FlashAdam):
@@ -114,11 +126,13 @@ class FlashAdamW(FlashAdam):
         master_weight_bits: Optional[Literal[24, 32]] = 24,
         check_numerics: bool = False,
         fused: bool = True,
+        *,
+        exact_update: Optional[bool] = None,
     ):
         super().__init__(
             params, lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, quantize=quantize,
             compress_state_dict=compress_state_dict, master_weight_bits=master_weight_bits,
-            check_numerics=check_numerics, fused=fused,
+            check_numerics=check_numerics, fused=fused, exact_update=exact_update,
         )
         self._decoupled = True
         self._decouple_lr = decouple_lr

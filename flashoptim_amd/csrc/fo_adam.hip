@@ -36,14 +36,13 @@ __device__ __forceinline__ void adam_load(const TensorPtrs& t, Where w, AdamRaw<
     }
 }
 
-template <int DT, int ECCB, bool QUANT, bool DECOUPLED, int FAST>
+template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT, int FAST>
 __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRaw<DT, ECCB, QUANT>& raw,
                                             const AdamHyper& h, const float* lut) {
     constexpr int EPL = DTypeInfo<DT>::epl;
     constexpr int PB = DTypeInfo<DT>::bytes;
     constexpr int SB = QUANT ? 1 : PB;
-    constexpr bool EXACT = AdamExact<DT, ECCB>::value;
-    constexpr bool MAY_BE_QUICK = QUANT && AdamQuickRequant<DT, ECCB>::value;  // fo_math.h: "two requantisers"
+    constexpr bool MAY_BE_QUICK = QUANT && !EXACT && AdamQuickRequant<DT, ECCB>::value;  // fo_math.h: "two requantisers"
     const int64_t n = t.n;
     const bool live_group = FAST == kVector || w.first() < n;  // the lane owns at least one real element
     const float sm = f16_bits_to_f32(raw.sm), sv = f16_bits_to_f32(raw.sv);
@@ -125,7 +124,9 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
     }
 }
 
-template <int DT, int ECCB, bool QUANT, bool DECOUPLED> struct AdamOp {
+// EXACT: the update follows the reference operation by operation (fo_math.h: AdamExact names the variants that do so
+// by default; the *_exact entry points ask for it on every variant).
+template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT = AdamExact<DT, ECCB>::value> struct AdamOp {
     using Hyper = AdamHyper;
     static constexpr int kLutTables = ECCB == 1 ? 2 : (QUANT ? 1 : 0);  // LDS code tables (fo_device.h)
     static constexpr int kDtype = DT;
@@ -133,7 +134,8 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED> struct AdamOp {
     // resident workgroups per compute unit for 2-byte parameters with no or a 1-byte ECC (3.6-4.1 KiB of loads per
     // wavefront; 13 and 16 are two to four points worse), 16 with a 2-byte ECC (4.6 KiB), 18-20 for fp32 parameters
     // (2.5 KiB)
-    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 20 : (ECCB == 2 ? 16 : 15);
+    // (the operation-by-operation update on 2-byte parameters is arithmetic-bound: as many as its registers allow)
+    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 20 : (EXACT ? 20 : (ECCB == 2 ? 16 : 15));
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {
@@ -141,7 +143,7 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED> struct AdamOp {
     }
     template <int FAST>
     __device__ __forceinline__ static void finish(const TensorPtrs& t, Where w, Raw& r, const Hyper& h, const float* lut) {
-        adam_finish<DT, ECCB, QUANT, DECOUPLED, FAST>(t, w, r, h, lut);
+        adam_finish<DT, ECCB, QUANT, DECOUPLED, EXACT, FAST>(t, w, r, h, lut);
     }
 };
 
@@ -152,6 +154,15 @@ using namespace fo_host;
 
 template <int DT, int EB, bool Q> using AdamL2Op = fo::AdamOp<DT, EB, Q, false>;  // FlashAdam: decay folded into the gradient
 template <int DT, int EB, bool Q> using AdamWOp = fo::AdamOp<DT, EB, Q, true>;    // FlashAdamW: decay applied to the weights
+template <int DT, int EB, bool Q> using AdamL2ExactOp = fo::AdamOp<DT, EB, Q, false, true>;
+template <int DT, int EB, bool Q> using AdamWExactOp = fo::AdamOp<DT, EB, Q, true, true>;
+
+template <class L> int dispatch_adam(int dtype, int ecc_bytes, int quantized, int decoupled, int exact, L&& launcher) {
+    if (exact)
+        return decoupled ? dispatch<AdamWExactOp>(dtype, ecc_bytes, quantized, launcher)
+                         : dispatch<AdamL2ExactOp>(dtype, ecc_bytes, quantized, launcher);
+    return decoupled ? dispatch<AdamWOp>(dtype, ecc_bytes, quantized, launcher) : dispatch<AdamL2Op>(dtype, ecc_bytes, quantized, launcher);
+}
 
 using fo::make_adam_hyper;
 
@@ -217,9 +228,9 @@ __global__ __launch_bounds__(256) void stage_tables_kernel(StageBatch b, fo_tens
 
 extern "C" {
 
-int fo_adam_step(void* mom, void* mom_scales, void* var, void* var_scales, void* param, const void* grad, void* ecc,
-                 int64_t n, int dtype, int ecc_bytes, int quantized, float lr, float beta1, float beta2, float eps,
-                 float weight_decay, int decoupled, int step, void* stream) {
+static int adam_step_any(void* mom, void* mom_scales, void* var, void* var_scales, void* param, const void* grad, void* ecc,
+                         int64_t n, int dtype, int ecc_bytes, int quantized, float lr, float beta1, float beta2, float eps,
+                         float weight_decay, int decoupled, int step, void* stream, int exact) {
     if (int rc = validate_common(param, grad, ecc, n, dtype, ecc_bytes)) return rc;
     if (n == 0) return 0;  // ref:2221-2223
     if (step < 1) return fail(FO_ERR_INVALID_ARGUMENT, "step must be >= 1 (got %d)", step);
@@ -227,17 +238,45 @@ int fo_adam_step(void* mom, void* mom_scales, void* var, void* var_scales, void*
     if (int rc = validate_state(var, var_scales, quantized, dtype, "var")) return rc;
     fo::TensorPtrs t{param, grad, ecc_bytes ? ecc : nullptr, mom, (uint16_t*)mom_scales, var, (uint16_t*)var_scales, n};
     SingleLauncher<fo::AdamHyper> L{t, make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step), (hipStream_t)stream};
-    return decoupled ? dispatch<AdamWOp>(dtype, ecc_bytes, quantized, L) : dispatch<AdamL2Op>(dtype, ecc_bytes, quantized, L);
+    return dispatch_adam(dtype, ecc_bytes, quantized, decoupled, exact, L);
+}
+
+int fo_adam_step(void* mom, void* mom_scales, void* var, void* var_scales, void* param, const void* grad, void* ecc,
+                 int64_t n, int dtype, int ecc_bytes, int quantized, float lr, float beta1, float beta2, float eps,
+                 float weight_decay, int decoupled, int step, void* stream) {
+    return adam_step_any(mom, mom_scales, var, var_scales, param, grad, ecc, n, dtype, ecc_bytes, quantized, lr, beta1, beta2,
+                         eps, weight_decay, decoupled, step, stream, 0);
+}
+
+int fo_adam_step_exact(void* mom, void* mom_scales, void* var, void* var_scales, void* param, const void* grad, void* ecc,
+                       int64_t n, int dtype, int ecc_bytes, int quantized, float lr, float beta1, float beta2, float eps,
+                       float weight_decay, int decoupled, int step, void* stream) {
+    return adam_step_any(mom, mom_scales, var, var_scales, param, grad, ecc, n, dtype, ecc_bytes, quantized, lr, beta1, beta2,
+                         eps, weight_decay, decoupled, step, stream, 1);
+}
+
+static int multi_adam_step_any(const fo_tensor_desc* descs, int64_t n_tensors, const fo_chunk* chunks, int64_t n_chunks,
+                               int dtype, int ecc_bytes, int quantized, float lr, float beta1, float beta2, float eps,
+                               float weight_decay, int decoupled, int step, void* stream, int exact) {
+    if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
+    if (n_chunks == 0) return 0;
+    if (step < 1) return fail(FO_ERR_INVALID_ARGUMENT, "step must be >= 1 (got %d)", step);
+    MultiLauncher<fo::AdamHyper> L{descs, chunks, n_chunks, make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step), (hipStream_t)stream};
+    return dispatch_adam(dtype, ecc_bytes, quantized, decoupled, exact, L);
 }
 
 int fo_multi_adam_step(const fo_tensor_desc* descs, int64_t n_tensors, const fo_chunk* chunks, int64_t n_chunks, int dtype,
                        int ecc_bytes, int quantized, float lr, float beta1, float beta2, float eps, float weight_decay,
                        int decoupled, int step, void* stream) {
-    if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
-    if (n_chunks == 0) return 0;
-    if (step < 1) return fail(FO_ERR_INVALID_ARGUMENT, "step must be >= 1 (got %d)", step);
-    MultiLauncher<fo::AdamHyper> L{descs, chunks, n_chunks, make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step), (hipStream_t)stream};
-    return decoupled ? dispatch<AdamWOp>(dtype, ecc_bytes, quantized, L) : dispatch<AdamL2Op>(dtype, ecc_bytes, quantized, L);
+    return multi_adam_step_any(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes, quantized, lr, beta1, beta2, eps,
+                               weight_decay, decoupled, step, stream, 0);
+}
+
+int fo_multi_adam_step_exact(const fo_tensor_desc* descs, int64_t n_tensors, const fo_chunk* chunks, int64_t n_chunks, int dtype,
+                             int ecc_bytes, int quantized, float lr, float beta1, float beta2, float eps, float weight_decay,
+                             int decoupled, int step, void* stream) {
+    return multi_adam_step_any(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes, quantized, lr, beta1, beta2, eps,
+                               weight_decay, decoupled, step, stream, 1);
 }
 
 int fo_multi_adam_step_static(const fo_tensor_desc* host_descs, int64_t n_tensors, int dtype, int ecc_bytes, int quantized,

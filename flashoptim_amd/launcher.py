@@ -177,9 +177,9 @@ class BucketPlan:
                     DTYPE_CODE[self.dtype], self.ecc_bytes, int(self.quantized))
             stream = _native.current_stream_ptr(self.device)
             if self.kind == "adam":
-                rc = lib.fo_multi_adam_step(*head, scalars["lr"], scalars["beta1"], scalars["beta2"], scalars["eps"],
-                                            scalars["weight_decay"], int(scalars["decoupled"]), int(scalars["step"]),
-                                            stream)
+                entry = lib.fo_multi_adam_step_exact if scalars.get("exact_update") else lib.fo_multi_adam_step
+                rc = entry(*head, scalars["lr"], scalars["beta1"], scalars["beta2"], scalars["eps"],
+                           scalars["weight_decay"], int(scalars["decoupled"]), int(scalars["step"]), stream)
             elif self.kind == "plain":
                 rc = lib.fo_multi_sgd_plain_step(*head[:6], scalars["lr"], scalars["weight_decay"],
                                                  int(scalars["decoupled"]), stream)

@@ -137,6 +137,24 @@ int fo_multi_adam_step_static(const fo_tensor_desc *host_descs, int64_t n_tensor
                               int quantized, float lr, float beta1, float beta2, float eps, float weight_decay,
                               int decoupled, int step, void *stream);
 
+/*
+ * fo_adam_step / fo_multi_adam_step with the update evaluated operation by operation as the reference writes it,
+ *     p -= (lr * (m / bc1)) / (sqrt(v / bc2) + eps)          (ref:2368-2375)
+ * with correctly rounded quotients and roots and the moments formed without folding (ref:2332-2360), for every
+ * parameter dtype.  Every output bit then equals an IEEE evaluation of the reference's formulas.  The plain entry
+ * points do this for fp32 parameters only; for bf16 / fp16 parameters they fold the bias corrections and the
+ * learning rate into two constants (one reciprocal per element), which leaves 1e-4 (24-bit masters) to 2e-2
+ * (32-bit masters) of the master weights more than one unit of master precision away from that evaluation, and is
+ * roughly 10-20 % faster.  Same arguments and errors as the plain entry points.  The reference has one kernel and no such
+ * choice; these are for callers who want the stricter arithmetic.
+ */
+int fo_adam_step_exact(void *mom, void *mom_scales, void *var, void *var_scales, void *param, const void *grad,
+                       void *ecc, int64_t n, int dtype, int ecc_bytes, int quantized, float lr, float beta1,
+                       float beta2, float eps, float weight_decay, int decoupled, int step, void *stream);
+int fo_multi_adam_step_exact(const fo_tensor_desc *descs, int64_t n_tensors, const fo_chunk *chunks,
+                             int64_t n_chunks, int dtype, int ecc_bytes, int quantized, float lr, float beta1,
+                             float beta2, float eps, float weight_decay, int decoupled, int step, void *stream);
+
 /* Momentum-free SGD over many tensors: the multi-tensor form of fo_sgd_plain_step (descs use param, grad, ecc, n). */
 int fo_multi_sgd_plain_step(const fo_tensor_desc *descs, int64_t n_tensors, const fo_chunk *chunks,
                             int64_t n_chunks, int dtype, int ecc_bytes, float lr, float weight_decay,

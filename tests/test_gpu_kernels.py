@@ -187,19 +187,21 @@ class _Case:
         return worst, beyond
 
 
-def _adam_steps(n, dtype, ecc_dtype, quantized, decoupled, steps, seed, offset=0, grad_scale=1e-3):
+def _adam_steps(n, dtype, ecc_dtype, quantized, decoupled, steps, seed, offset=0, grad_scale=1e-3, exact_update=False):
     """Returns per step (code mismatch fraction, fraction of master weights beyond one unit)."""
     k = _k()
     c = _Case(n, dtype, ecc_dtype, quantized, 2, seed, offset)
     lr, b1, b2, eps = 1e-3, 0.9, 0.999, 1e-8
     wd = 0.01 * lr if decoupled else 0.01
-    exact = dtype == torch.float32  # fp32 parameters: the update follows the reference operation by operation
+    # fp32 parameters, or exact_update: the update follows the reference operation by operation
+    exact = dtype == torch.float32 or exact_update
     out = []
     for step in range(1, steps + 1):
         g = _rand(n, grad_scale, 1000 * seed + step).to(dtype)
         gg = c._dev(g)
         (m, ms), (v, vs) = c.gstates
-        k._fused_adam_step(m, ms, v, vs, c.gp, gg, c.gecc, lr, b1, b2, eps, wd, decoupled, step, quantize_optim_states=quantized)
+        k._fused_adam_step(m, ms, v, vs, c.gp, gg, c.gecc, lr, b1, b2, eps, wd, decoupled, step, quantize_optim_states=quantized,
+                           exact_update=exact_update)
         info = T.adam_step_ref(c.states[0], c.states[1], c.p, g, c.ecc, lr, b1, b2, eps, wd, decoupled, step)
         out.append(c.compare(f"adam n={n} {dtype} ecc={ecc_dtype} q={quantized} step={step}", info, exact))
         c.resync_oracle()
@@ -215,6 +217,17 @@ def test_adam_step_matches_oracle(dtype, ecc_dtype, quantized, decoupled):
         # the first step starts from zero states: m and v are formed exactly as the reference forms them and the
         # requantiser follows its rounding, so not a single code may differ
         assert stats[0][0] == 0.0, f"first-step codes differ (n={n})"
+
+
+@pytest.mark.parametrize("dtype,ecc_dtype", [v for v in VARIANTS if v[0] != torch.float32])
+@pytest.mark.parametrize("quantized", [True, False])
+@pytest.mark.parametrize("decoupled", [True, False])
+def test_adam_exact_update_is_bit_exact_for_narrow_parameters(dtype, ecc_dtype, quantized, decoupled):
+    """fo_adam_step_exact: the operation-by-operation update on bf16 / fp16 parameters.  Every output bit of every
+    step equals the oracle's (parameters, ECC, codes, scales), as for fp32 parameters."""
+    for i, n in enumerate([1, 31, 33, 1000, 4097 + 4096, (1 << 16) + 17]):
+        _adam_steps(n, dtype, ecc_dtype, quantized, decoupled, steps=4, seed=i + 1, exact_update=True)
+    _adam_steps(5000, dtype, ecc_dtype, quantized, decoupled, steps=3, seed=9, offset=3, exact_update=True)
 
 
 @pytest.mark.parametrize("ecc_dtype", [torch.int8, torch.int16])

@@ -96,6 +96,48 @@ def test_config0_loss_trajectory_matches_oracle():
         assert (st["exp_avg"].quantized.cpu().reshape(-1).int() - s["m"].codes.int()).abs().float().mean() < 1.0
 
 
+@pytest.mark.parametrize("bits,ecc_dtype", [(24, torch.int8), (32, torch.int16)])
+def test_config0_with_exact_update_equals_the_oracle_bit_for_bit(bits, ecc_dtype):
+    """FlashAdamW(exact_update=True) on the README MLP (bf16 parameters; one multi-tensor launch per step through
+    fo_multi_adam_step_exact), free running for 50 steps next to the oracle-stepped copy: the losses are equal and
+    in the end every parameter, ECC code, moment code and scale is the oracle's, bit for bit."""
+    fo = _fo()
+    x = torch.randn(32, 128, generator=torch.Generator().manual_seed(0)).to(DEV, torch.bfloat16)
+    model_a, model_b = _mlp().to(DEV), _mlp().to(DEV)
+    fo.cast_model(model_a)
+    fo.cast_model(model_b)
+    hp = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+    opt_a = fo.FlashAdamW(model_a.parameters(), master_weight_bits=bits, exact_update=True, **hp)
+    opt_b = OracleAdamW(model_b.parameters(), ecc_dtype=ecc_dtype, **hp)
+    for step in range(50):
+        losses = []
+        for model, opt in ((model_a, opt_a), (model_b, opt_b)):
+            for p in model.parameters():
+                p.grad = None
+            loss = model(x).float().sum()
+            loss.backward()
+            opt.step()
+            losses.append(loss.item())
+        assert losses[0] == losses[1], f"step {step}: loss {losses[0]} vs oracle {losses[1]}"
+    for p, s in zip(model_a.parameters(), opt_b.state):
+        st = opt_a.state[p]
+        assert parity.bits_equal(p.detach().reshape(-1), s["p"])
+        assert parity.bits_equal(st["error_bits"].reshape(-1), s["ecc"])
+        assert parity.bits_equal(st["exp_avg"].quantized.reshape(-1), s["m"].codes)
+        assert parity.bits_equal(st["exp_avg"].scales.reshape(-1)[:s["m"].scales.numel()], s["m"].scales)
+        assert parity.bits_equal(st["exp_avg_sq"].quantized.reshape(-1), s["v"].codes)
+        assert parity.bits_equal(st["exp_avg_sq"].scales.reshape(-1)[:s["v"].scales.numel()], s["v"].scales)
+
+
+def test_exact_update_defaults_to_the_environment_variable(monkeypatch):
+    fo = _fo()
+    p = [nn.Parameter(torch.zeros(8, dtype=torch.bfloat16, device=DEV))]
+    assert fo.FlashAdamW(p)._exact_update is False
+    monkeypatch.setenv("FLASHOPTIM_EXACT_ADAM", "1")
+    assert fo.FlashAdamW(p)._exact_update is True
+    assert fo.FlashAdam(p, exact_update=False)._exact_update is False
+
+
 # ------------------------------------------------------------------------------ multi-tensor launcher
 
 _RAGGED = [1, 31, 32, 33, 1000, 4096, 4097, 12289, 70001, 3, 262144 + 7]

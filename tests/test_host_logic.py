@@ -160,8 +160,12 @@ def test_public_names_match_the_reference_package():
     import inspect
 
     sig = inspect.signature(FlashAdamW.__init__)
+    # the reference's parameters in its order; the one addition is keyword-only and defaults to off
     assert list(sig.parameters)[1:] == ["params", "lr", "betas", "eps", "weight_decay", "decouple_lr", "quantize",
-                                        "compress_state_dict", "master_weight_bits", "check_numerics", "fused"]
+                                        "compress_state_dict", "master_weight_bits", "check_numerics", "fused",
+                                        "exact_update"]
+    assert sig.parameters["exact_update"].kind is inspect.Parameter.KEYWORD_ONLY
+    assert sig.parameters["exact_update"].default is None
     assert sig.parameters["weight_decay"].default == 1e-2 and sig.parameters["master_weight_bits"].default == 24
     sig = inspect.signature(FlashLion.__init__)
     assert sig.parameters["betas"].default == (0.9, 0.99) and sig.parameters["weight_decay"].default == 0
