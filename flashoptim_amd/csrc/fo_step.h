@@ -8,7 +8,7 @@
 // that each touch every stream once than with larger or persistent ones.  The multi-tensor grid addresses work
 // through a chunk table in units of 4096-element tiles; a tile is an integer number of spans.  A quantisation
 // group is 32/EPL neighbouring lanes, so the group absmax is in-register maxes plus two or three DPP moves.
-// LDS only holds the table that turns a first-moment code byte into its dequantised value.
+// LDS only holds the two 256-entry code tables (first-moment code -> value, int8 ECC code -> fraction).
 //
 // "ref:" cites /root/reference/flashoptim/optimizers.py.
 #pragma once
