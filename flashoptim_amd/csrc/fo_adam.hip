@@ -77,15 +77,6 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
     store_lane<ECCB, EPL, FAST>(eout, t.ecc, w, n);
 
     if constexpr (QUANT) {
-        // wavefront-uniform: one group of the span that starts from a zero state sends the whole span through the
-        // exact requantiser
-        const bool quick = MAY_BE_QUICK && __builtin_amdgcn_ballot_w64(scale_is_zero(raw.sm) || scale_is_zero(raw.sv)) == 0;
-        if constexpr (MAY_BE_QUICK) {
-            if (!quick) {
-#pragma unroll
-                for (int k = 0; k < EPL; ++k) r[k] = sqrt_corrected(v[k]);
-            }
-        }
         float am = 0.0f, av = 0.0f;
 #pragma unroll
         for (int k = 0; k < EPL; k += 2) {  // pairs, so that each step is one three-operand max
@@ -95,6 +86,22 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
         // group absmax (ref:2399-2404)
         am = fmaxf(group_max<EPL>(am), 1e-12f);
         av = fmaxf(group_max<EPL>(av), 1e-12f);
+        // wavefront-uniform choice of the requantiser: one group of the span whose old state is zero, or dwarfed by
+        // the new second moment (quick_requant_allowed), sends the whole span through the exact forms
+        bool quick = false;
+        if constexpr (MAY_BE_QUICK) {
+            quick = __builtin_amdgcn_ballot_w64(!quick_requant_allowed(raw.sm, raw.sv, sv, av)) == 0;
+            if (!quick) {
+                av = 0.0f;
+#pragma unroll
+                for (int k = 0; k < EPL; k += 2) {
+                    r[k] = sqrt_corrected(v[k]);
+                    r[k + 1] = sqrt_corrected(v[k + 1]);
+                    av = fmaxf(fmaxf(av, r[k]), r[k + 1]);
+                }
+                av = fmaxf(group_max<EPL>(av), 1e-12f);
+            }
+        }
         if constexpr (MAY_BE_QUICK) {
             static_assert(EPL == 8, "2-byte parameters");
             if (quick) {

@@ -233,8 +233,8 @@ FO_FN float quantize_var_rounded(float r, float av, float rav) {
 // The quick forms are the same real-number formulas with the quotients merged and approximate (a few ulps), the
 // rounding still floor(x + 0.5).  Adam on 2-byte parameters with no or a 1-byte ECC (AdamQuickRequant; its update
 // is folded and therefore already agrees with the reference to rounding error only, see adam_apply) uses them for
-// every wavefront span in which no group starts from a zero state (scale_is_zero); a span with such a group, and
-// every other kernel, uses the exact forms.  rav255 = 255 * rcp(group maximum of sqrt(v)); the quick path takes
+// every wavefront span in which no group starts from a zero or negligible state (quick_requant_allowed); a span
+// with such a group, and every other kernel, uses the exact forms.  rav255 = 255 * rcp(group maximum of sqrt(v)); the quick path takes
 // sqrt(v) from hw::sqrt.
 FO_FN float quantize_mom_quick(float m, float am) {
     const float t = m * hw::rcp(am + fabsf(m));  // = nm / (1 + |nm|), nm = m / am
@@ -243,6 +243,18 @@ FO_FN float quantize_mom_quick(float m, float am) {
 FO_FN float quantize_var_quick(float r, float rav255) { return hw::fma(r, rav255, 0.5f); }
 // A stored fp16 group scale of zero: every element of the group is zero (ref:2399-2404 store the absmax).
 FO_FN bool scale_is_zero(uint16_t f16_bits) { return (f16_bits & 0x7fffu) == 0; }
+// May a group take the quick forms?  Not from a zero state (either scale zero), and not when the new second moment
+// dwarfs the old one: sv_old is the old group maximum of sqrt(v), av_new the new one (from hw::sqrt).  The share
+// of the old state in the new v is about (sv_old / av_new)^2; once it falls below 1e-4 the new values sit within
+// a few hundred ulps of the near-ties they would have from a zero state, and the quick forms' own few ulps pick
+// the other code on more than 1e-4 of the elements (measured on the CPU build with a sudden jump of the gradient
+// scale: 3e-5 of the codes at a share of 1e-4, 2e-4 at 1e-5, 4e-3 below 1e-7).  The bound used is a share of 1e-3
+// (av_new > 32 sv_old: a gradient a thousand times the group's running maximum once v has converged, thirty-odd
+// times during the first steps).  The first moment has no such regime short of a 1e8-fold jump: its old value
+// enters with weight beta1 / (1 - beta1), not with the square of a ratio.
+FO_FN bool quick_requant_allowed(uint16_t sm_bits, uint16_t sv_bits, float sv_old, float av_new) {
+    return !scale_is_zero(sm_bits) && !scale_is_zero(sv_bits) && !(av_new > 32.0f * sv_old);
+}
 FO_FN u32 quantize_mom_code(float m, float am, float ram) { return (u32)hw::floor_to_int(quantize_mom_rounded(m, am, ram)); }
 FO_FN u32 quantize_var_code(float r, float av, float rav) { return (u32)(int)quantize_var_rounded(r, av, rav); }
 

@@ -81,80 +81,83 @@ template <int DT, int ECCB> void write_master(void* param, void* ecc, int64_t i,
     if constexpr (ECCB > 0) store_ecc<ECCB>(ecc, i, ecc_split_bits<DT, ECCB, false>(p, w));
 }
 
-// the structure of adam_finish (fo_adam.hip), one quantisation group at a time; QUICK as the kernel's template
-// argument of that name
-template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT, bool QUICK>
-void adam_group(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scales, void* param, const void* grad, void* ecc,
-                int64_t n, int64_t g0, const AdamHyper& h) {
-    const int cnt = (int)((n - g0) < kGroup ? (n - g0) : kGroup);
-    const int64_t group = g0 >> 5;
-    float sm = 1.0f, sv = 1.0f;
-    if (QUANT) { sm = f16_to_f32(mom_scales[group]); sv = f16_to_f32(var_scales[group]); }
-    const float sm_b1 = sm * h.b1, sv_b2 = sv * h.sqrt_b2_over_255;
-    float m[kGroup], r[kGroup], v[kGroup];
-    float am = 0.0f, av = 0.0f;
-    for (int k = 0; k < cnt; ++k) {
-        const int64_t i = g0 + k;
-        float p = read_master<DT, ECCB>(param, ecc, i);
-        float gr = load_elem<DT>(grad, i);
-        if (!DECOUPLED) gr = gr + p * h.wd;
-        float mn, vn;
-        if (QUANT) {
-            adam_moments_quantized<EXACT>(gr, kTable.v[((const uint8_t*)mom)[i]], sm, sm_b1, (float)((const uint8_t*)var)[i],
-                                          sv, sv_b2, h, mn, vn);
-        } else {
-            adam_moments_plain(gr, load_elem<DT>(mom, i), load_elem<DT>(var, i), h, mn, vn);
-        }
-        if (DECOUPLED) p = p * h.one_m_wd;
-        constexpr bool kMayBeQuick = QUANT && !EXACT && AdamQuickRequant<DT, ECCB>::value;
-        float rk = (QUANT || !EXACT) ? (kMayBeQuick ? hw::sqrt(vn) : sqrt_corrected(vn)) : 0.0f;
-        p = adam_apply<EXACT>(p, mn, vn, rk, h);
-        write_master<DT, ECCB>(param, ecc, i, p);
-        if (kMayBeQuick && !QUICK) rk = sqrt_corrected(vn);  // the exact requantiser wants the correctly rounded root
-        m[k] = mn; r[k] = rk; v[k] = vn;
-        am = fmaxf(am, fabsf(mn));
-        av = fmaxf(av, rk);
-    }
-    if (QUANT) {
-        am = fmaxf(am, 1e-12f);
-        av = fmaxf(av, 1e-12f);
-        const float ram = hw::rcp(am), rav = hw::rcp(av);
-        const float rav255 = rav * 255.0f;
-        for (int k = 0; k < cnt; ++k) {
-            if (QUICK) {
-                ((uint8_t*)mom)[g0 + k] = (uint8_t)hw::floor_to_int(quantize_mom_quick(m[k], am));
-                ((uint8_t*)var)[g0 + k] = (uint8_t)(int)quantize_var_quick(r[k], rav255);
-            } else {
-                ((uint8_t*)mom)[g0 + k] = (uint8_t)quantize_mom_code(m[k], am, ram);
-                ((uint8_t*)var)[g0 + k] = (uint8_t)quantize_var_code(r[k], av, rav);
-            }
-        }
-        mom_scales[group] = f32_to_f16(am);
-        var_scales[group] = f32_to_f16(av);
-    } else {
-        for (int k = 0; k < cnt; ++k) {
-            store_elem<DT>(mom, g0 + k, m[k]);
-            store_elem<DT>(var, g0 + k, v[k]);
-        }
-    }
-}
-
-// One wavefront span (64 lanes x EPL elements, counted from the start of the tensor) at a time: like the kernel, a
-// span takes the quick requantiser unless one of its groups starts from a zero state.
+// the structure of adam_finish (fo_adam.hip), one wavefront span (64 lanes x EPL elements, counted from the start of
+// the tensor) at a time and one quantisation group at a time inside it: first the update of every group, with
+// sqrt(v) as the folded update takes it; then, like the kernel, the span-wide choice of the requantiser
+// (quick_requant_allowed for every group, else the exact forms on correctly rounded roots); then the codes.
 template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT>
 void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scales, void* param, const void* grad, void* ecc,
                  int64_t n, const AdamHyper& h) {
     constexpr int64_t kSpan = 64 * DTypeInfo<DT>::epl;
+    constexpr int kGroupsPerSpan = (int)(kSpan / kGroup);
     constexpr bool kMayBeQuick = QUANT && !EXACT && AdamQuickRequant<DT, ECCB>::value;
+    struct GroupWork { float m[kGroup], r[kGroup], v[kGroup], am, av; int cnt; };
+    static thread_local GroupWork work[kGroupsPerSpan];
     for (int64_t s0 = 0; s0 < n; s0 += kSpan) {
         const int64_t s1 = (s0 + kSpan) < n ? (s0 + kSpan) : n;
         bool quick = kMayBeQuick;
-        if (kMayBeQuick)
-            for (int64_t g0 = s0; g0 < s1; g0 += kGroup)
-                if (scale_is_zero(mom_scales[g0 >> 5]) || scale_is_zero(var_scales[g0 >> 5])) quick = false;
-        for (int64_t g0 = s0; g0 < s1; g0 += kGroup) {
-            if (quick) adam_group<DT, ECCB, QUANT, DECOUPLED, EXACT, kMayBeQuick>(mom, mom_scales, var, var_scales, param, grad, ecc, n, g0, h);
-            else adam_group<DT, ECCB, QUANT, DECOUPLED, EXACT, false>(mom, mom_scales, var, var_scales, param, grad, ecc, n, g0, h);
+        int n_groups = 0;
+        for (int64_t g0 = s0; g0 < s1; g0 += kGroup, ++n_groups) {
+            GroupWork& w = work[n_groups];
+            w.cnt = (int)((n - g0) < kGroup ? (n - g0) : kGroup);
+            const int64_t group = g0 >> 5;
+            float sm = 1.0f, sv = 1.0f;
+            if (QUANT) { sm = f16_to_f32(mom_scales[group]); sv = f16_to_f32(var_scales[group]); }
+            const float sm_b1 = sm * h.b1, sv_b2 = sv * h.sqrt_b2_over_255;
+            w.am = 0.0f; w.av = 0.0f;
+            for (int k = 0; k < w.cnt; ++k) {
+                const int64_t i = g0 + k;
+                float p = read_master<DT, ECCB>(param, ecc, i);
+                float gr = load_elem<DT>(grad, i);
+                if (!DECOUPLED) gr = gr + p * h.wd;
+                float mn, vn;
+                if (QUANT) {
+                    adam_moments_quantized<EXACT>(gr, kTable.v[((const uint8_t*)mom)[i]], sm, sm_b1,
+                                                  (float)((const uint8_t*)var)[i], sv, sv_b2, h, mn, vn);
+                } else {
+                    adam_moments_plain(gr, load_elem<DT>(mom, i), load_elem<DT>(var, i), h, mn, vn);
+                }
+                if (DECOUPLED) p = p * h.one_m_wd;
+                const float rk = (QUANT || !EXACT) ? (kMayBeQuick ? hw::sqrt(vn) : sqrt_corrected(vn)) : 0.0f;
+                p = adam_apply<EXACT>(p, mn, vn, rk, h);
+                write_master<DT, ECCB>(param, ecc, i, p);
+                w.m[k] = mn; w.r[k] = rk; w.v[k] = vn;
+                w.am = fmaxf(w.am, fabsf(mn));
+                w.av = fmaxf(w.av, rk);
+            }
+            w.am = fmaxf(w.am, 1e-12f);
+            w.av = fmaxf(w.av, 1e-12f);
+            if (kMayBeQuick && !quick_requant_allowed(mom_scales[group], var_scales[group], sv, w.av)) quick = false;
+        }
+        int gi = 0;
+        for (int64_t g0 = s0; g0 < s1; g0 += kGroup, ++gi) {
+            GroupWork& w = work[gi];
+            const int64_t group = g0 >> 5;
+            if (!QUANT) {
+                for (int k = 0; k < w.cnt; ++k) {
+                    store_elem<DT>(mom, g0 + k, w.m[k]);
+                    store_elem<DT>(var, g0 + k, w.v[k]);
+                }
+                continue;
+            }
+            if (kMayBeQuick && !quick) {  // the exact requantiser wants the correctly rounded roots and their maximum
+                w.av = 0.0f;
+                for (int k = 0; k < w.cnt; ++k) { w.r[k] = sqrt_corrected(w.v[k]); w.av = fmaxf(w.av, w.r[k]); }
+                w.av = fmaxf(w.av, 1e-12f);
+            }
+            const float ram = hw::rcp(w.am), rav = hw::rcp(w.av);
+            const float rav255 = rav * 255.0f;
+            for (int k = 0; k < w.cnt; ++k) {
+                if (kMayBeQuick && quick) {
+                    ((uint8_t*)mom)[g0 + k] = (uint8_t)hw::floor_to_int(quantize_mom_quick(w.m[k], w.am));
+                    ((uint8_t*)var)[g0 + k] = (uint8_t)(int)quantize_var_quick(w.r[k], rav255);
+                } else {
+                    ((uint8_t*)mom)[g0 + k] = (uint8_t)quantize_mom_code(w.m[k], w.am, ram);
+                    ((uint8_t*)var)[g0 + k] = (uint8_t)quantize_var_code(w.r[k], w.av, rav);
+                }
+            }
+            mom_scales[group] = f32_to_f16(w.am);
+            var_scales[group] = f32_to_f16(w.av);
         }
     }
 }

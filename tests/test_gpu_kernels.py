@@ -271,6 +271,27 @@ def test_adam_groups_that_start_from_zero_get_the_exact_requantiser(dtype, ecc_d
         assert torch.equal(a.cpu()[in_reset], s.codes[in_reset]), "a group that started from zero differs from the oracle"
 
 
+def test_adam_sudden_jump_of_the_gradient_scale_keeps_the_code_tolerance():
+    """Three steps at gradient scale 1e-4, then one step with gradients 1 to 1e5 times larger: the old second moment
+    becomes negligible, the new values sit near rounding boundaries as on a first step, and the kernel must fall
+    back to the exact requantiser for such groups (quick forms alone: up to 0.4 % of the codes off)."""
+    k = _k()
+    n = (1 << 18) + 5
+    lr, b1, b2, eps, wd = 1e-3, 0.9, 0.999, 1e-8, 1e-5
+    for jump in (1.0, 10.0, 30.0, 100.0, 1e3, 1e5):
+        c = _Case(n, torch.bfloat16, torch.int8, True, 2, seed=3)
+        (m, ms), (v, vs) = c.gstates
+        for step in (1, 2, 3):
+            g = _rand(n, 1e-4, 10 + step).to(torch.bfloat16)
+            k._fused_adam_step(m, ms, v, vs, c.gp, g.to(DEV), c.gecc, lr, b1, b2, eps, wd, True, step, quantize_optim_states=True)
+        c.resync_oracle()
+        g = _rand(n, 1e-4 * jump, 99).to(torch.bfloat16)
+        k._fused_adam_step(m, ms, v, vs, c.gp, g.to(DEV), c.gecc, lr, b1, b2, eps, wd, True, 4, quantize_optim_states=True)
+        info = T.adam_step_ref(c.states[0], c.states[1], c.p, g, c.ecc, lr, b1, b2, eps, wd, True, 4)
+        worst, _ = c.compare(f"adam after a {jump:g}-fold gradient jump", info, exact=False)
+        print(f"jump {jump:g}: code mismatch {worst:.1e}")
+
+
 def test_adam_unaligned_pointers():
     _adam_steps(5000, torch.bfloat16, torch.int8, True, True, steps=3, seed=9, offset=3)
     _adam_steps(5000, torch.float32, None, True, True, steps=3, seed=9, offset=1)
