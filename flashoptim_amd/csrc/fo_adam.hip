@@ -87,10 +87,10 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
         am = fmaxf(group_max<EPL>(am), 1e-12f);
         av = fmaxf(group_max<EPL>(av), 1e-12f);
         // wavefront-uniform choice of the requantiser: one group of the span whose old state is zero, or dwarfed by
-        // the new second moment (quick_requant_allowed), sends the whole span through the exact forms
+        // the new moments (quick_requant_allowed), sends the whole span through the exact forms
         bool quick = false;
         if constexpr (MAY_BE_QUICK) {
-            quick = __builtin_amdgcn_ballot_w64(!quick_requant_allowed(raw.sm, raw.sv, sv, av)) == 0;
+            quick = __builtin_amdgcn_ballot_w64(!quick_requant_allowed(raw.sm, raw.sv, sm_b1, am, sv_b2, av)) == 0;
             if (!quick) {
                 av = 0.0f;
 #pragma unroll

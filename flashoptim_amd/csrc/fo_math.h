@@ -243,17 +243,21 @@ FO_FN float quantize_mom_quick(float m, float am) {
 FO_FN float quantize_var_quick(float r, float rav255) { return hw::fma(r, rav255, 0.5f); }
 // A stored fp16 group scale of zero: every element of the group is zero (ref:2399-2404 store the absmax).
 FO_FN bool scale_is_zero(uint16_t f16_bits) { return (f16_bits & 0x7fffu) == 0; }
-// May a group take the quick forms?  Not from a zero state (either scale zero), and not when the new second moment
-// dwarfs the old one: sv_old is the old group maximum of sqrt(v), av_new the new one (from hw::sqrt).  The share
-// of the old state in the new v is about (sv_old / av_new)^2; once it falls below 1e-4 the new values sit within
-// a few hundred ulps of the near-ties they would have from a zero state, and the quick forms' own few ulps pick
-// the other code on more than 1e-4 of the elements (measured on the CPU build with a sudden jump of the gradient
-// scale: 3e-5 of the codes at a share of 1e-4, 2e-4 at 1e-5, 4e-3 below 1e-7).  The bound used is a share of 1e-3
-// (av_new > 32 sv_old: a gradient a thousand times the group's running maximum once v has converged, thirty-odd
-// times during the first steps).  The first moment has no such regime short of a 1e8-fold jump: its old value
-// enters with weight beta1 / (1 - beta1), not with the square of a ratio.
-FO_FN bool quick_requant_allowed(uint16_t sm_bits, uint16_t sv_bits, float sv_old, float av_new) {
-    return !scale_is_zero(sm_bits) && !scale_is_zero(sv_bits) && !(av_new > 32.0f * sv_old);
+// May a group take the quick forms?  Not from a zero state (either scale zero), and not when the new moments dwarf
+// what the old state contributes to them.  Arguments besides the scale bits: sm_b1 = old first-moment scale (the
+// old group maximum of |m|) times beta1, am_new = new group maximum of |m|; sv_b2 = old second-moment scale (the old
+// group maximum of sqrt(v)) times sqrt(beta2) / 255 as the folded form carries it, av_new = the new group maximum
+// of sqrt(v) (from hw::sqrt).  The share of the old state in the new v is about (sv_old sqrt(beta2) / av_new)^2;
+// once it falls below 1e-4 the new values sit within a few hundred ulps of the near-ties they would have from a
+// zero state, and the quick forms' own few ulps pick the other code on more than 1e-4 of the elements (measured on
+// the CPU build with a sudden jump of the gradient scale: 3e-5 of the codes at a share of 1e-4, 2e-4 at 1e-5, 4e-3
+// below 1e-7).  The bound used is a share of 1e-3 for either moment: av_new > 32 sv_old sqrt(beta2) (a gradient a
+// thousand times the group's running maximum once v has converged, thirty-odd times during the first steps), or
+// am_new > 1024 sm_old beta1.  beta1 = 0 or beta2 = 0 (no memory at all: every step is a first step) therefore
+// always take the exact forms.
+FO_FN bool quick_requant_allowed(uint16_t sm_bits, uint16_t sv_bits, float sm_b1, float am_new, float sv_b2, float av_new) {
+    return !scale_is_zero(sm_bits) && !scale_is_zero(sv_bits) && !(am_new > 1024.0f * sm_b1) &&
+           !(av_new > (32.0f * 255.0f) * sv_b2);
 }
 FO_FN u32 quantize_mom_code(float m, float am, float ram) { return (u32)hw::floor_to_int(quantize_mom_rounded(m, am, ram)); }
 FO_FN u32 quantize_var_code(float r, float av, float rav) { return (u32)(int)quantize_var_rounded(r, av, rav); }

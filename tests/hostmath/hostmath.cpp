@@ -127,7 +127,7 @@ void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scale
             }
             w.am = fmaxf(w.am, 1e-12f);
             w.av = fmaxf(w.av, 1e-12f);
-            if (kMayBeQuick && !quick_requant_allowed(mom_scales[group], var_scales[group], sv, w.av)) quick = false;
+            if (kMayBeQuick && !quick_requant_allowed(mom_scales[group], var_scales[group], sm_b1, w.am, sv_b2, w.av)) quick = false;
         }
         int gi = 0;
         for (int64_t g0 = s0; g0 < s1; g0 += kGroup, ++gi) {

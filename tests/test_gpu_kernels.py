@@ -292,6 +292,22 @@ def test_adam_sudden_jump_of_the_gradient_scale_keeps_the_code_tolerance():
         print(f"jump {jump:g}: code mismatch {worst:.1e}")
 
 
+@pytest.mark.parametrize("betas", [(0.0, 0.999), (0.9, 0.0), (0.0, 0.0), (0.01, 0.999), (0.9, 0.1), (0.5, 0.9), (0.99, 0.9999)])
+def test_adam_code_tolerance_holds_for_unusual_betas(betas):
+    """beta1 = 0 or beta2 = 0: the old state has no weight and every step is as tie-prone as a first step; the
+    kernel must keep such steps on the exact requantiser."""
+    k = _k()
+    n = (1 << 18) + 5
+    c = _Case(n, torch.bfloat16, torch.int8, True, 2, seed=3)
+    (m, ms), (v, vs) = c.gstates
+    for step in range(1, 5):
+        g = _rand(n, 1e-3, 10 + step).to(torch.bfloat16)
+        k._fused_adam_step(m, ms, v, vs, c.gp, g.to(DEV), c.gecc, 1e-3, betas[0], betas[1], 1e-8, 1e-5, True, step, quantize_optim_states=True)
+        info = T.adam_step_ref(c.states[0], c.states[1], c.p, g, c.ecc, 1e-3, betas[0], betas[1], 1e-8, 1e-5, True, step)
+        c.compare(f"adam betas {betas} step {step}", info, exact=False)
+        c.resync_oracle()
+
+
 def test_adam_unaligned_pointers():
     _adam_steps(5000, torch.bfloat16, torch.int8, True, True, steps=3, seed=9, offset=3)
     _adam_steps(5000, torch.float32, None, True, True, steps=3, seed=9, offset=1)

@@ -279,6 +279,23 @@ def test_a_sudden_jump_of_the_gradient_scale_keeps_the_code_tolerance(noise):
             parity.check_codes(a[key], b[key], f"jump {jump:g} {key}")
 
 
+@pytest.mark.parametrize("betas", [(0.0, 0.999), (0.9, 0.0), (0.0, 0.0), (0.01, 0.999), (0.9, 0.1), (0.5, 0.9), (0.99, 0.9999)])
+def test_code_tolerance_holds_for_unusual_betas(betas):
+    """beta1 = 0 or beta2 = 0 make every step a first step for that moment (the old state has no weight, the new
+    values are a narrow gradient times a constant); small betas come close.  The choice of the requantiser looks at
+    what the old state contributes, not only at whether it is zero."""
+    H.set_noise(7)
+    n = 1 << 17
+    a = _adam_state(n, torch.bfloat16, torch.int8, True, seed=3)
+    for step in range(1, 5):
+        g = _rand(n, 1e-3, 10 + step).to(torch.bfloat16)
+        b = _clone(a)
+        T.adam_step_ref(T.MomentState(b["m"], b["ms"]), T.MomentState(b["v"], b["vs"]), b["p"], g, b["e"], 1e-3, betas[0], betas[1], 1e-8, 1e-5, True, step)
+        H.adam_step(a["m"], a["ms"], a["v"], a["vs"], a["p"], g, a["e"], 1e-3, betas[0], betas[1], 1e-8, 1e-5, True, step)
+        for key in ("m", "v"):
+            parity.check_codes(a[key], b[key], f"betas {betas} step {step} {key}")
+
+
 def test_master_weight_error_of_the_folded_update_without_allowance():
     """How far the folded Adam update strays from the reference's operation order, with no allowance: the share of
     master weights more than one unit of master precision away from the oracle's (weights ~N(0, 0.02), gradients
