@@ -43,21 +43,24 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
     constexpr int PB = DTypeInfo<DT>::bytes;
     constexpr int SB = QUANT ? 1 : PB;
     constexpr bool MAY_BE_QUICK = QUANT && !EXACT && AdamQuickRequant<DT, ECCB>::value;  // fo_math.h: "two requantisers"
+    constexpr bool EXACT_MOMENTS = EXACT || !AdamFoldedMoments<DT, ECCB>::value;
     const int64_t n = t.n;
     const bool live_group = FAST == kVector || w.first() < n;  // the lane owns at least one real element
     const float sm = f16_bits_to_f32(raw.sm), sv = f16_bits_to_f32(raw.sv);
     const float sm_b1 = sm * h.b1, sv_b2 = sv * h.sqrt_b2_over_255;
 
     float p[EPL], m[EPL], r[EPL], v[EPL];
+    float gmax = 0.0f;  // largest |g| of the lane (the requantiser choice asks whether it sets the new scales alone)
     read_master<DT, ECCB, EPL>(p, raw.p, raw.e, lut);
 
 #pragma unroll
     for (int k = 0; k < EPL; ++k) {
         float g = widen<DT, EPL>(raw.g, k);
         if constexpr (!DECOUPLED) g = g + p[k] * h.wd;                              // ref:2310-2311
+        if constexpr (MAY_BE_QUICK) gmax = fmaxf(gmax, fabsf(g));
         float mn, vn;
         if constexpr (QUANT) {
-            adam_moments_quantized<EXACT>(g, lookup_mom(lut, byte_of<EPL>(raw.m, k)), sm, sm_b1,
+            adam_moments_quantized<EXACT_MOMENTS>(g, lookup_mom(lut, byte_of<EPL>(raw.m, k)), sm, sm_b1,
                                           (float)byte_of<EPL>(raw.v, k), sv, sv_b2, h, mn, vn);
         } else {
             adam_moments_plain(g, widen<DT, EPL>(raw.m, k), widen<DT, EPL>(raw.v, k), h, mn, vn);
@@ -84,13 +87,15 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
             av = fmaxf(fmaxf(av, r[k]), r[k + 1]);
         }
         // group absmax (ref:2399-2404)
-        am = fmaxf(group_max<EPL>(am), 1e-12f);
-        av = fmaxf(group_max<EPL>(av), 1e-12f);
-        // wavefront-uniform choice of the requantiser: one group of the span whose old state is zero, or dwarfed by
-        // the new moments (quick_requant_allowed), sends the whole span through the exact forms
+        am = group_max<EPL>(am);
+        av = group_max<EPL>(av);
+        // wavefront-uniform choice of the requantiser: one group of the span whose new maxima carry no old state
+        // (quick_requant_allowed) sends the whole span through the exact forms
         bool quick = false;
         if constexpr (MAY_BE_QUICK) {
-            quick = __builtin_amdgcn_ballot_w64(!quick_requant_allowed(raw.sm, raw.sv, sm_b1, am, sv_b2, av)) == 0;
+            gmax = group_max<EPL>(gmax);
+            quick = __builtin_amdgcn_ballot_w64(!quick_requant_allowed(raw.sm, raw.sv, sm_b1, am, sv_b2, av, gmax, h.one_m_b1,
+                                                                       h.one_m_b2)) == 0;
             if (!quick) {
                 av = 0.0f;
 #pragma unroll
@@ -99,9 +104,11 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
                     r[k + 1] = sqrt_corrected(v[k + 1]);
                     av = fmaxf(fmaxf(av, r[k]), r[k + 1]);
                 }
-                av = fmaxf(group_max<EPL>(av), 1e-12f);
+                av = group_max<EPL>(av);
             }
         }
+        am = fmaxf(am, 1e-12f);
+        av = fmaxf(av, 1e-12f);
         if constexpr (MAY_BE_QUICK) {
             static_assert(EPL == 8, "2-byte parameters");
             if (quick) {

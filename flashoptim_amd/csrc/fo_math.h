@@ -231,7 +231,7 @@ FO_FN float quantize_var_rounded(float r, float av, float rav) {
 // the old state contributes, the values are generic and a formula that is a few ulps off picks another code only
 // for the 1e-5 of the elements whose value lies within those ulps of a boundary.
 // The quick forms are the same real-number formulas with the quotients merged and approximate (a few ulps), the
-// rounding still floor(x + 0.5).  Adam on 2-byte parameters with no or a 1-byte ECC (AdamQuickRequant; its update
+// rounding still floor(x + 0.5).  Adam on bf16 parameters with no or a 1-byte ECC (AdamQuickRequant; its update
 // is folded and therefore already agrees with the reference to rounding error only, see adam_apply) uses them for
 // every wavefront span in which no group starts from a zero or negligible state (quick_requant_allowed); a span
 // with such a group, and every other kernel, uses the exact forms.  rav255 = 255 * rcp(group maximum of sqrt(v)); the quick path takes
@@ -243,21 +243,30 @@ FO_FN float quantize_mom_quick(float m, float am) {
 FO_FN float quantize_var_quick(float r, float rav255) { return hw::fma(r, rav255, 0.5f); }
 // A stored fp16 group scale of zero: every element of the group is zero (ref:2399-2404 store the absmax).
 FO_FN bool scale_is_zero(uint16_t f16_bits) { return (f16_bits & 0x7fffu) == 0; }
-// May a group take the quick forms?  Not from a zero state (either scale zero), and not when the new moments dwarf
-// what the old state contributes to them.  Arguments besides the scale bits: sm_b1 = old first-moment scale (the
-// old group maximum of |m|) times beta1, am_new = new group maximum of |m|; sv_b2 = old second-moment scale (the old
-// group maximum of sqrt(v)) times sqrt(beta2) / 255 as the folded form carries it, av_new = the new group maximum
-// of sqrt(v) (from hw::sqrt).  The share of the old state in the new v is about (sv_old sqrt(beta2) / av_new)^2;
-// once it falls below 1e-4 the new values sit within a few hundred ulps of the near-ties they would have from a
-// zero state, and the quick forms' own few ulps pick the other code on more than 1e-4 of the elements (measured on
-// the CPU build with a sudden jump of the gradient scale: 3e-5 of the codes at a share of 1e-4, 2e-4 at 1e-5, 4e-3
-// below 1e-7).  The bound used is a share of 1e-3 for either moment: av_new > 32 sv_old sqrt(beta2) (a gradient a
-// thousand times the group's running maximum once v has converged, thirty-odd times during the first steps), or
-// am_new > 1024 sm_old beta1.  beta1 = 0 or beta2 = 0 (no memory at all: every step is a first step) therefore
-// always take the exact forms.
-FO_FN bool quick_requant_allowed(uint16_t sm_bits, uint16_t sv_bits, float sm_b1, float am_new, float sv_b2, float av_new) {
-    return !scale_is_zero(sm_bits) && !scale_is_zero(sv_bits) && !(am_new > 1024.0f * sm_b1) &&
-           !(av_new > (32.0f * 255.0f) * sv_b2);
+// May a group take the quick forms?  Only if its new maxima carry old state.  The exact forms matter where a code's
+// pre-rounding value 255 r / av (or its first-moment counterpart) is a ratio of two "simple" numbers, each a
+// narrow-precision gradient times a constant: 0.3 % of such ratios sit exactly on a rounding boundary.  An
+// element's value is simple when its own old state is zero or negligible; the ratio is simple only if the group
+// maximum is simple too.  So the question is asked of the maxima:
+//   * either old scale zero: the whole group starts from zero;
+//   * the new maximum equals what the largest gradient of the group gives from a zero state, to the bit
+//     (am_new == gmax (1 - beta1), av_new == sqrt(gmax^2 (1 - beta2)), evaluated with the very operations the
+//     update uses): the element that sets the scale had a zero old state (its old code was 0: sparse gradients,
+//     or the first steps, where 0.3 % of the codes are 0);
+//   * the old state's share in the new maximum is below 1e-3: av_new > 32 sv_old sqrt(beta2), i.e. a gradient a
+//     thousand times the group's running maximum once v has converged and thirty-odd times during the first steps,
+//     or am_new > 1024 sm_old beta1 (measured on the CPU build with a sudden jump of the gradient scale: the quick
+//     forms pick the other code on 3e-5 of the elements at a share of 1e-4, 2e-4 at 1e-5, 4e-3 below 1e-7).
+//     beta1 = 0 or beta2 = 0 (no memory at all: every step is a first step) fall under this rule.
+// Arguments: the old scales' bits; sm_b1 = old first-moment scale times beta1; sv_b2 = old second-moment scale times
+// sqrt(beta2) / 255 (as the folded form carries them); am_new, av_new = new group maxima of |m| and of sqrt(v) (the
+// latter from hw::sqrt), before their clamp; gmax = group maximum of |g| (g as it enters the moments).
+FO_FN bool quick_requant_allowed(uint16_t sm_bits, uint16_t sv_bits, float sm_b1, float am_new, float sv_b2, float av_new,
+                                 float gmax, float one_m_b1, float one_m_b2) {
+    const bool from_zero = scale_is_zero(sm_bits) || scale_is_zero(sv_bits);
+    const bool pure_max = am_new == gmax * one_m_b1 || av_new == hw::sqrt((gmax * gmax) * one_m_b2);
+    const bool dwarfed = am_new > 1024.0f * sm_b1 || av_new > (32.0f * 255.0f) * sv_b2;
+    return !(from_zero || pure_max || dwarfed);
 }
 FO_FN u32 quantize_mom_code(float m, float am, float ram) { return (u32)hw::floor_to_int(quantize_mom_rounded(m, am, ram)); }
 FO_FN u32 quantize_var_code(float r, float av, float rav) { return (u32)(int)quantize_var_rounded(r, av, rav); }
@@ -308,9 +317,18 @@ inline AdamHyper make_adam_hyper(float lr, float beta1, float beta2, float eps, 
 // fp32 parameters, where one fp32 ulp is the master precision and the 16.25 bytes per element leave room
 // for the extra arithmetic.  Narrow parameters use the folded update (see adam_apply).
 template <int DT, int ECCB> struct AdamExact { static constexpr bool value = DT == DT_F32; };
-// Variants whose wavefronts may take the quick requantiser: those with the folded update, except the ones with a
-// 2-byte ECC, whose 14.25 bytes per element hide the exact requantiser's arithmetic (measured: no gain).
-template <int DT, int ECCB> struct AdamQuickRequant { static constexpr bool value = !AdamExact<DT, ECCB>::value && ECCB != 2; };
+// Variants that form the new moments with the decay folded into the group scale (adam_moments_quantized): bf16
+// parameters.  fp16 parameters keep the reference's operation order for the moments although their update is
+// folded: fp16 gradients underflow into a handful of subnormal values, moments built from so few distinct values
+// sit exactly on rounding boundaries in bulk, and the folded form's one-ulp differences then move up to 1e-2 of
+// the codes; with the unfolded moments and the exact requantiser their codes and scales equal the oracle's always.
+template <int DT, int ECCB> struct AdamFoldedMoments { static constexpr bool value = DT == DT_BF16; };
+// Variants whose wavefronts may take the quick requantiser: bf16 parameters with the folded update and no or a
+// 1-byte ECC.  Not with a 2-byte ECC, whose 14.25 bytes per element hide the exact requantiser's arithmetic
+// (measured: no gain).  Not fp16 parameters: their small gradients are fp16 subnormals, a handful of multiples of
+// 2^-24, and moments built from so few distinct values sit on rounding boundaries in bulk whatever the old state
+// is (measured: 1e-2 of the codes).
+template <int DT, int ECCB> struct AdamQuickRequant { static constexpr bool value = DT == DT_BF16 && ECCB != 2; };
 
 // New moments from the dequantised pieces.
 //   EXACT = false: the EMA decay is folded into the group scale (one multiply per lane instead of one per

@@ -91,7 +91,7 @@ void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scale
     constexpr int64_t kSpan = 64 * DTypeInfo<DT>::epl;
     constexpr int kGroupsPerSpan = (int)(kSpan / kGroup);
     constexpr bool kMayBeQuick = QUANT && !EXACT && AdamQuickRequant<DT, ECCB>::value;
-    struct GroupWork { float m[kGroup], r[kGroup], v[kGroup], am, av; int cnt; };
+    struct GroupWork { float m[kGroup], r[kGroup], v[kGroup], am, av, gmax; int cnt; };
     static thread_local GroupWork work[kGroupsPerSpan];
     for (int64_t s0 = 0; s0 < n; s0 += kSpan) {
         const int64_t s1 = (s0 + kSpan) < n ? (s0 + kSpan) : n;
@@ -104,15 +104,16 @@ void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scale
             float sm = 1.0f, sv = 1.0f;
             if (QUANT) { sm = f16_to_f32(mom_scales[group]); sv = f16_to_f32(var_scales[group]); }
             const float sm_b1 = sm * h.b1, sv_b2 = sv * h.sqrt_b2_over_255;
-            w.am = 0.0f; w.av = 0.0f;
+            w.am = 0.0f; w.av = 0.0f; w.gmax = 0.0f;
             for (int k = 0; k < w.cnt; ++k) {
                 const int64_t i = g0 + k;
                 float p = read_master<DT, ECCB>(param, ecc, i);
                 float gr = load_elem<DT>(grad, i);
                 if (!DECOUPLED) gr = gr + p * h.wd;
+                w.gmax = fmaxf(w.gmax, fabsf(gr));
                 float mn, vn;
                 if (QUANT) {
-                    adam_moments_quantized<EXACT>(gr, kTable.v[((const uint8_t*)mom)[i]], sm, sm_b1,
+                    adam_moments_quantized<(EXACT || !AdamFoldedMoments<DT, ECCB>::value)>(gr, kTable.v[((const uint8_t*)mom)[i]], sm, sm_b1,
                                                   (float)((const uint8_t*)var)[i], sv, sv_b2, h, mn, vn);
                 } else {
                     adam_moments_plain(gr, load_elem<DT>(mom, i), load_elem<DT>(var, i), h, mn, vn);
@@ -125,9 +126,10 @@ void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scale
                 w.am = fmaxf(w.am, fabsf(mn));
                 w.av = fmaxf(w.av, rk);
             }
+            if (kMayBeQuick && !quick_requant_allowed(mom_scales[group], var_scales[group], sm_b1, w.am, sv_b2, w.av, w.gmax,
+                                                       h.one_m_b1, h.one_m_b2))
+                quick = false;
             w.am = fmaxf(w.am, 1e-12f);
-            w.av = fmaxf(w.av, 1e-12f);
-            if (kMayBeQuick && !quick_requant_allowed(mom_scales[group], var_scales[group], sm_b1, w.am, sv_b2, w.av)) quick = false;
         }
         int gi = 0;
         for (int64_t g0 = s0; g0 < s1; g0 += kGroup, ++gi) {
@@ -143,8 +145,8 @@ void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scale
             if (kMayBeQuick && !quick) {  // the exact requantiser wants the correctly rounded roots and their maximum
                 w.av = 0.0f;
                 for (int k = 0; k < w.cnt; ++k) { w.r[k] = sqrt_corrected(w.v[k]); w.av = fmaxf(w.av, w.r[k]); }
-                w.av = fmaxf(w.av, 1e-12f);
             }
+            w.av = fmaxf(w.av, 1e-12f);
             const float ram = hw::rcp(w.am), rav = hw::rcp(w.av);
             const float rav255 = rav * 255.0f;
             for (int k = 0; k < w.cnt; ++k) {

@@ -163,7 +163,9 @@ class _Case:
 
     def compare(self, what, info, exact):
         """`info`: the oracle's intermediates of the step just taken.  exact: every output bit must equal the
-        oracle's (all kernels but Adam on bf16 / fp16 parameters, see tests/parity.py).
+        oracle's (all kernels but Adam on bf16 / fp16 parameters, see tests/parity.py).  fp16 parameters under Adam:
+        the update is folded (master weights within tolerance) but the moments are not, so codes and scales must be
+        the oracle's bit for bit.
         Returns (worst code mismatch fraction, fraction of master weights beyond one unit with no allowance)."""
         if exact:
             assert parity.bits_equal(self.gp, self.p), f"{what}: parameter bits differ"
@@ -179,7 +181,10 @@ class _Case:
         _, beyond = parity.check_master(self.gp, self.gecc, self.p, self.ecc, what, step_size=info["update_scale"])
         worst = 0.0
         for i, (s, (a, b)) in enumerate(zip(self.states, self.gstates)):
-            if self.quantized:
+            if self.quantized and self.dtype == torch.float16:
+                assert parity.bits_equal(a, s.codes), f"{what} state{i}: fp16 codes differ"
+                assert parity.bits_equal(b, s.scales), f"{what} state{i}: fp16 scales differ"
+            elif self.quantized:
                 worst = max(worst, parity.check_codes(a, s.codes, f"{what} state{i}"))
                 parity.check_scales(b, s.scales, f"{what} state{i}")
             else:
