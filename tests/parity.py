@@ -4,9 +4,11 @@ What the kernels promise (flashoptim_amd/csrc/fo_math.h) and what the tests ther
 identical inputs:
 * SGD / SGDW / Nesterov / Lion steps, the momentum-free SGD step, Adam with fp32 parameters, unquantised states, the
   standalone codec and the standalone ECC kernels: every output bit equals the oracle's (`bits_equal`);
-* Adam with bf16 / fp16 parameters (folded update): the new moments come out of fused multiply-adds and may differ
-  from the oracle's by an ulp, and wavefront spans in which every group carries a state that the new gradient
-  does not dwarf requantise with the quick forms (a few ulps off; no or 1-byte ECC only), so
+* Adam with fp16 parameters (folded update, unfolded moments): codes and scales bit-exact, master weights and
+  narrow parameters as in the next item;
+* Adam with bf16 parameters (folded update and moments): the new moments come out of fused multiply-adds and may
+  differ from the oracle's by an ulp, and wavefront spans in which every group's new maxima carry old state
+  requantise with the quick forms (a few ulps off; no or 1-byte ECC only), so
   - 8-bit moment codes never differ by more than +-1 code step and differ on fewer than 0.01 % of the elements
     (measured 1e-6 .. 2.5e-5; exactly 0 on a first step from zero states and in any group that starts from zero,
     where m and v are formed identically and the exact requantiser runs);
