@@ -313,6 +313,28 @@ def test_adam_code_tolerance_holds_for_unusual_betas(betas):
         c.resync_oracle()
 
 
+@pytest.mark.parametrize("dtype,exact_update", [(torch.bfloat16, True), (torch.float16, False)])
+def test_adam_on_lattice_valued_gradients_stays_bit_exact_where_promised(dtype, exact_update):
+    """Sign gradients of one magnitude and gradients that are small integer multiples of a unit keep the moments on a
+    coarse lattice whose ratios (1/2, 1/3, ...) sit exactly on rounding boundaries in bulk.  The paths that promise
+    bit-exact codes on any data must deliver them here: bf16 parameters with the operation-by-operation update
+    (every output bit) and fp16 parameters by default (codes and scales; their moments are formed unfolded)."""
+    k = _k()
+    n = (1 << 16) + 9
+    lr, b1, b2, eps, wd = 1e-3, 0.5, 0.95, 1e-8, 1e-5
+    for kind in ("sign", "integers"):
+        c = _Case(n, dtype, torch.int8, True, 2, seed=4)
+        (m, ms), (v, vs) = c.gstates
+        for step, unit in enumerate((2e-3, 2e-3, 20.0, 20.0, 2e-3), start=1):
+            z = _rand(n, 1.0, 300 + step)
+            g = (torch.sign(z) * unit if kind == "sign" else torch.round(z) * unit).to(dtype)
+            k._fused_adam_step(m, ms, v, vs, c.gp, g.to(DEV), c.gecc, lr, b1, b2, eps, wd, True, step, quantize_optim_states=True,
+                               exact_update=exact_update)
+            info = T.adam_step_ref(c.states[0], c.states[1], c.p, g, c.ecc, lr, b1, b2, eps, wd, True, step)
+            c.compare(f"adam {dtype} {kind} gradients step {step}", info, exact=exact_update)
+            c.resync_oracle()
+
+
 def test_adam_unaligned_pointers():
     _adam_steps(5000, torch.bfloat16, torch.int8, True, True, steps=3, seed=9, offset=3)
     _adam_steps(5000, torch.float32, None, True, True, steps=3, seed=9, offset=1)
