@@ -148,8 +148,8 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT = AdamExact<D
     // resident workgroups per compute unit for 2-byte parameters with no or a 1-byte ECC (3.6-4.1 KiB of loads per
     // wavefront; 13 and 16 are two to four points worse), 16 with a 2-byte ECC (4.6 KiB), 18-20 for fp32 parameters
     // (2.5 KiB)
-    // (the operation-by-operation update on 2-byte parameters is arithmetic-bound: as many as its registers allow)
-    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 20 : (EXACT ? 20 : (ECCB == 2 ? 16 : 15));
+    // (the operation-by-operation update on 2-byte parameters is arithmetic-bound: what its 90-99 VGPRs allow)
+    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 20 : (ECCB == 2 || EXACT ? 16 : 15);
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {
