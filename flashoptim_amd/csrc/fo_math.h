@@ -223,19 +223,17 @@ FO_FN float quantize_var_rounded(float r, float av, float rav) {
     return q * 255.0f + 0.5f;  // non-negative: truncation is the floor
 }
 // Two requantisers.  The exact one above costs two corrected quotients per first-moment value and a corrected
-// quotient plus a corrected square root per second-moment value.  What it buys shows where the pre-rounding value
-// of a code lies on a rounding boundary k + 1/2 to the last bit, and that happens in bulk only when the new
-// moments are a narrow-precision gradient times a constant, i.e. when the old state of the group is zero (first
-// step, or a group whose gradients have been zero so far): 0.3 % of the second-moment values of such a group sit
-// exactly on a boundary, and which side they fall on depends on every rounding of the reference's formula.  Once
-// the old state contributes, the values are generic and a formula that is a few ulps off picks another code only
-// for the 1e-5 of the elements whose value lies within those ulps of a boundary.
-// The quick forms are the same real-number formulas with the quotients merged and approximate (a few ulps), the
-// rounding still floor(x + 0.5).  Adam on bf16 parameters with no or a 1-byte ECC (AdamQuickRequant; its update
-// is folded and therefore already agrees with the reference to rounding error only, see adam_apply) uses them for
-// every wavefront span in which no group starts from a zero or negligible state (quick_requant_allowed); a span
-// with such a group, and every other kernel, uses the exact forms.  rav255 = 255 * rcp(group maximum of sqrt(v)); the quick path takes
-// sqrt(v) from hw::sqrt.
+// quotient plus a corrected square root per second-moment value.  The quick forms below are the same real-number
+// formulas with the quotients merged and approximate (a few ulps), the rounding still floor(x + 0.5).  For values
+// drawn from a continuum a few ulps move the code of about 1e-5 of the elements, those within that distance of a
+// rounding boundary.  They fail where values sit on a boundary to the last bit in bulk, which quick_requant_allowed
+// (below) detects for the cases that arise with continuous gradients; gradients confined to a handful of
+// magnitudes for a whole run (sign gradients, integer multiples of a unit) keep all moments on a lattice and are
+// beyond it (up to 1e-3 of the codes off by one step, far more in constructed cases).
+// Adam on bf16 parameters with no or a 1-byte ECC (AdamQuickRequant; its update is folded and therefore already
+// agrees with the reference to rounding error only, see adam_apply) uses the quick forms for every wavefront span
+// whose groups all pass quick_requant_allowed; a span with a group that does not, and every other kernel, uses the
+// exact forms.  rav255 = 255 * rcp(group maximum of sqrt(v)); the quick path takes sqrt(v) from hw::sqrt.
 FO_FN float quantize_mom_quick(float m, float am) {
     const float t = m * hw::rcp(am + fabsf(m));  // = nm / (1 + |nm|), nm = m / am
     return hw::fma(t, 254.0f, 0.5f);
