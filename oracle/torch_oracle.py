@@ -93,7 +93,10 @@ def quantize_groups(
     groups, n = _group_view(x_f32)
     if sqrt:
         groups = _sqrt_rn(groups)
-    absmax = groups.abs().amax(dim=1).clamp_min(f32(1e-12))
+    # tl.max / tl.maximum (ref:2657-2658) are NaN-ignoring reductions (Triton's default): a NaN element does not
+    # poison its group's scale
+    mags = groups.abs()
+    absmax = torch.where(torch.isnan(mags), torch.zeros_like(mags), mags).amax(dim=1).clamp_min(f32(1e-12))
     normalized = groups / absmax[:, None]
     if softsign:
         transformed = (2.0 * normalized) / (1.0 + normalized.abs())

@@ -177,3 +177,17 @@ def test_fp16_scale_conversion_exhaustive_slices():
     allh = np.arange(0, 0x7C01, dtype=np.uint16)
     back = np.array([lib.fo_oracle_f16_to_f32(int(h)) for h in allh[::7]], dtype=np.float32)
     assert np.array_equal(back, allh[::7].view(np.float16).astype(np.float32))
+
+
+def test_a_nan_element_does_not_poison_its_groups_scale():
+    """The reference's group maximum is `tl.max` followed by `tl.maximum(., 1e-12)` (ref:2657-2658), NaN-ignoring
+    reductions: a NaN element leaves the scale of its group to the other 31.  Both restatements agree on that (the
+    code stored for the NaN element itself is unspecified and not compared)."""
+    x = torch.linspace(-2.0, 3.0, 96)
+    x[40] = float("nan")
+    _, scales_t = T.quantize_ref(x, True, False, True)
+    _, scales_c = C.quantize(x, True, False, True)
+    assert torch.equal(scales_t, scales_c) and not bool(torch.isnan(scales_t.float()).any())
+    assert scales_t[1] == x[32:64][~torch.isnan(x[32:64])].abs().max().to(torch.float16)
+    all_nan = torch.full((32,), float("nan"))
+    assert T.quantize_ref(all_nan, True, False, True)[1][0] == torch.tensor(1e-12).to(torch.float16)
