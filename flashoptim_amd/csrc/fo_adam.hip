@@ -50,14 +50,12 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
     const float sm_b1 = sm * h.b1, sv_b2 = sv * h.sqrt_b2_over_255;
 
     float p[EPL], m[EPL], r[EPL], v[EPL];
-    float gmax = 0.0f;  // largest |g| of the lane (the requantiser choice asks whether it sets the new scales alone)
     read_master<DT, ECCB, EPL>(p, raw.p, raw.e, lut);
 
 #pragma unroll
     for (int k = 0; k < EPL; ++k) {
         float g = widen<DT, EPL>(raw.g, k);
         if constexpr (!DECOUPLED) g = g + p[k] * h.wd;                              // ref:2310-2311
-        if constexpr (MAY_BE_QUICK) gmax = fmaxf(gmax, fabsf(g));
         float mn, vn;
         if constexpr (QUANT) {
             adam_moments_quantized<EXACT_MOMENTS>(g, lookup_mom(lut, byte_of<EPL>(raw.m, k)), sm, sm_b1,
@@ -67,8 +65,8 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
         }
         float pk = p[k];
         if constexpr (DECOUPLED) pk = pk * h.one_m_wd;                              // ref:2363-2364
-        // sqrt(v): the requantiser needs it (ref:2393) and the folded update shares it.  The folded update is content
-        // with the instruction's value; the exact requantiser replaces it by the correctly rounded one below.
+        // sqrt(v): the requantiser needs it (ref:2393) and the folded update shares it.  The folded update and the
+        // quick requantiser forms are content with the instruction's value.
         const float rk = (QUANT || !EXACT) ? (MAY_BE_QUICK ? hw::sqrt(vn) : sqrt_corrected(vn)) : 0.0f;
         p[k] = adam_apply<EXACT>(pk, mn, vn, rk, h);                                // ref:2368-2375
         m[k] = mn; r[k] = rk; v[k] = vn;
@@ -80,48 +78,28 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
     store_lane<ECCB, EPL, FAST>(eout, t.ecc, w, n);
 
     if constexpr (QUANT) {
+        // group absmax (ref:2399-2404); the square root is monotone, so the largest sqrt(v) is the root of the largest v
         float am = 0.0f, av = 0.0f;
 #pragma unroll
         for (int k = 0; k < EPL; k += 2) {  // pairs, so that each step is one three-operand max
             am = fmaxf(fmaxf(am, fabsf(m[k])), fabsf(m[k + 1]));
-            av = fmaxf(fmaxf(av, r[k]), r[k + 1]);
+            if constexpr (MAY_BE_QUICK) av = fmaxf(fmaxf(av, v[k]), v[k + 1]);
+            else av = fmaxf(fmaxf(av, r[k]), r[k + 1]);
         }
-        // group absmax (ref:2399-2404)
-        am = group_max<EPL>(am);
+        am = fmaxf(group_max<EPL>(am), 1e-12f);
         av = group_max<EPL>(av);
-        // wavefront-uniform choice of the requantiser: one group of the span whose new maxima carry no old state
-        // (quick_requant_allowed) sends the whole span through the exact forms
-        bool quick = false;
-        if constexpr (MAY_BE_QUICK) {
-            gmax = group_max<EPL>(gmax);
-            quick = __builtin_amdgcn_ballot_w64(!quick_requant_allowed(raw.sm, raw.sv, sm_b1, am, sv_b2, av, gmax, h.one_m_b1,
-                                                                       h.one_m_b2)) == 0;
-            if (!quick) {
-                av = 0.0f;
-#pragma unroll
-                for (int k = 0; k < EPL; k += 2) {
-                    r[k] = sqrt_corrected(v[k]);
-                    r[k + 1] = sqrt_corrected(v[k + 1]);
-                    av = fmaxf(fmaxf(av, r[k]), r[k + 1]);
-                }
-                av = group_max<EPL>(av);
-            }
-        }
-        am = fmaxf(am, 1e-12f);
-        av = fmaxf(av, 1e-12f);
         if constexpr (MAY_BE_QUICK) {
             static_assert(EPL == 8, "2-byte parameters");
-            if (quick) {
-                quantize_mom<EPL, true>(m, am, raw.m);
-                quantize_var<EPL, true>(r, av, raw.v);
-            } else {
-                quantize_mom<EPL, false>(m, am, raw.m);
-                quantize_var<EPL, false>(r, av, raw.v);
-            }
+            const float av_quick = fmaxf(hw::sqrt(av), 1e-12f);   // av holds the group's largest v here
+            av = fmaxf(sqrt_corrected(av), 1e-12f);               // what the exact requantiser divides by, and the scale
+            quantize_mom_quick_verified<EPL>(m, am, raw.m);
+            quantize_var_quick_verified<EPL>(v, r, av_quick, av, raw.v);
         } else if constexpr (EPL == 8) {
+            av = fmaxf(av, 1e-12f);
             quantize_mom<EPL>(m, am, raw.m);
             quantize_var<EPL>(r, av, raw.v);
         } else {
+            av = fmaxf(av, 1e-12f);
             quantize_mom_var(m, am, r, av, raw.m, raw.v);
         }
         store_lane<1, EPL, FAST>(raw.m, t.mom, w, n);
@@ -144,12 +122,12 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT = AdamExact<D
     using Hyper = AdamHyper;
     static constexpr int kLutTables = ECCB == 1 ? 2 : (QUANT ? 1 : 0);  // LDS code tables (fo_device.h)
     static constexpr int kDtype = DT;
-    // measured on MI355X with the 8B-parameter step and this file's ILP-oriented instruction schedule: 14-15
-    // resident workgroups per compute unit for 2-byte parameters with no or a 1-byte ECC (3.6-4.1 KiB of loads per
-    // wavefront; 13 and 16 are two to four points worse), 16 with a 2-byte ECC (4.6 KiB), 18-20 for fp32 parameters
-    // (2.5 KiB)
-    // (the operation-by-operation update on 2-byte parameters is arithmetic-bound: what its 90-99 VGPRs allow)
-    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 20 : (ECCB == 2 || EXACT ? 16 : 15);
+    // measured on MI355X with the 8B-parameter step and this file's ILP-oriented instruction schedule: 16-17
+    // resident workgroups per compute unit for 2-byte parameters (3.6-4.6 KiB of loads per wavefront; 15 and 18
+    // are two to three points worse on the 8B list, a flat tensor does not care between 15 and 17), 18-20 for fp32
+    // parameters (2.5 KiB).  The operation-by-operation update on 2-byte parameters is arithmetic-bound and gets
+    // what its 90-99 VGPRs allow.
+    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 20 : 16;
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {

@@ -65,6 +65,7 @@ static inline float nudge(float exact, float x) {
 static inline float rcp(float x) { return nudge((float)(1.0 / (double)x), x); }
 static inline float rsq(float x) { return nudge((float)(1.0 / sqrt((double)x)), x); }
 static inline float sqrt(float x) { return nudge(sqrtf(x), x); }
+static inline float fract(float x) { return x - floorf(x); }
 static inline float ldexp(float x, int e) { return ldexpf(x, e); }
 static inline float med3(float x, float lo, float hi) { return fminf(fmaxf(x, lo), hi); }
 static inline int floor_to_int(float x) { return (int)floorf(x); }
@@ -73,6 +74,7 @@ static inline float fma(float a, float b, float c) { return __builtin_fmaf(a, b,
 FO_FN float rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 FO_FN float rsq(float x) { return __builtin_amdgcn_rsqf(x); }
 FO_FN float sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
+FO_FN float fract(float x) { return __builtin_amdgcn_fractf(x); }  // x - floor(x)
 FO_FN float ldexp(float x, int e) { return __builtin_amdgcn_ldexpf(x, e); }
 FO_FN float med3(float x, float lo, float hi) { return __builtin_amdgcn_fmed3f(x, lo, hi); }
 // (int)floor(x) in one instruction
@@ -222,52 +224,46 @@ FO_FN float quantize_var_rounded(float r, float av, float rav) {
     const float q = div_corrected(r, av, rav);
     return q * 255.0f + 0.5f;  // non-negative: truncation is the floor
 }
-// Two requantisers.  The exact one above costs two corrected quotients per first-moment value and a corrected
-// quotient plus a corrected square root per second-moment value.  The quick forms below are the same real-number
-// formulas with the quotients merged and approximate (a few ulps), the rounding still floor(x + 0.5).  For values
-// drawn from a continuum a few ulps move the code of about 1e-5 of the elements, those within that distance of a
-// rounding boundary.  They fail where values sit on a boundary to the last bit in bulk, which quick_requant_allowed
-// (below) detects for the cases that arise with continuous gradients; gradients confined to a handful of
-// magnitudes for a whole run (sign gradients, integer multiples of a unit) keep all moments on a lattice and are
-// beyond it (up to 1e-3 of the codes off by one step, far more in constructed cases).
-// Adam on bf16 parameters with no or a 1-byte ECC (AdamQuickRequant; its update is folded and therefore already
-// agrees with the reference to rounding error only, see adam_apply) uses the quick forms for every wavefront span
-// whose groups all pass quick_requant_allowed; a span with a group that does not, and every other kernel, uses the
-// exact forms.  rav255 = 255 * rcp(group maximum of sqrt(v)); the quick path takes sqrt(v) from hw::sqrt.
-FO_FN float quantize_mom_quick(float m, float am) {
-    const float t = m * hw::rcp(am + fabsf(m));  // = nm / (1 + |nm|), nm = m / am
-    return hw::fma(t, 254.0f, 0.5f);
-}
-FO_FN float quantize_var_quick(float r, float rav255) { return hw::fma(r, rav255, 0.5f); }
-// A stored fp16 group scale of zero: every element of the group is zero (ref:2399-2404 store the absmax).
-FO_FN bool scale_is_zero(uint16_t f16_bits) { return (f16_bits & 0x7fffu) == 0; }
-// May a group take the quick forms?  Only if its new maxima carry old state.  The exact forms matter where a code's
-// pre-rounding value 255 r / av (or its first-moment counterpart) is a ratio of two "simple" numbers, each a
-// narrow-precision gradient times a constant: 0.3 % of such ratios sit exactly on a rounding boundary.  An
-// element's value is simple when its own old state is zero or negligible; the ratio is simple only if the group
-// maximum is simple too.  So the question is asked of the maxima:
-//   * either old scale zero: the whole group starts from zero;
-//   * the new maximum equals what the largest gradient of the group gives from a zero state, to the bit
-//     (am_new == gmax (1 - beta1), av_new == sqrt(gmax^2 (1 - beta2)), evaluated with the very operations the
-//     update uses): the element that sets the scale had a zero old state (its old code was 0: sparse gradients,
-//     or the first steps, where 0.3 % of the codes are 0);
-//   * the old state's share in the new maximum is below 1e-3: av_new > 32 sv_old sqrt(beta2), i.e. a gradient a
-//     thousand times the group's running maximum once v has converged and thirty-odd times during the first steps,
-//     or am_new > 1024 sm_old beta1 (measured on the CPU build with a sudden jump of the gradient scale: the quick
-//     forms pick the other code on 3e-5 of the elements at a share of 1e-4, 2e-4 at 1e-5, 4e-3 below 1e-7).
-//     beta1 = 0 or beta2 = 0 (no memory at all: every step is a first step) fall under this rule.
-// Arguments: the old scales' bits; sm_b1 = old first-moment scale times beta1; sv_b2 = old second-moment scale times
-// sqrt(beta2) / 255 (as the folded form carries them); am_new, av_new = new group maxima of |m| and of sqrt(v) (the
-// latter from hw::sqrt), before their clamp; gmax = group maximum of |g| (g as it enters the moments).
-FO_FN bool quick_requant_allowed(uint16_t sm_bits, uint16_t sv_bits, float sm_b1, float am_new, float sv_b2, float av_new,
-                                 float gmax, float one_m_b1, float one_m_b2) {
-    const bool from_zero = scale_is_zero(sm_bits) || scale_is_zero(sv_bits);
-    const bool pure_max = am_new == gmax * one_m_b1 || av_new == hw::sqrt((gmax * gmax) * one_m_b2);
-    const bool dwarfed = am_new > 1024.0f * sm_b1 || av_new > (32.0f * 255.0f) * sv_b2;
-    return !(from_zero || pure_max || dwarfed);
-}
 FO_FN u32 quantize_mom_code(float m, float am, float ram) { return (u32)hw::floor_to_int(quantize_mom_rounded(m, am, ram)); }
 FO_FN u32 quantize_var_code(float r, float av, float rav) { return (u32)(int)quantize_var_rounded(r, av, rav); }
+// The quick forms.  The exact requantiser above costs two corrected quotients per first-moment value and a corrected
+// quotient plus a corrected square root per second-moment value.  The quick forms evaluate the same real-number
+// formulas with the quotients merged and approximate, and say whether their result can be trusted:
+//     first moment   x = 254 m / (am + |m|) + 0.5            as  fma(m * rcp(am + |m|), 254, 0.5 + margin)
+//     second moment  x = 255 r / av + 0.5                     as  fma(r, 255 * rcp(av), 0.5 + margin), r, av from hw::sqrt
+// Either form and the exact one stay within a known distance of the real-number value x (each rounding contributes
+// 2^-24 relative, each approximate instruction at most an ulp; in code units, with |x| <= 128 resp. 256):
+//     first moment   exact 3.8e-5, quick 3.8e-5   ->  they can differ by 7.6e-5   ->  margin 2^-13 = 1.2e-4
+//     second moment  exact 7.6e-5, quick 1.2e-4   ->  they can differ by 2.0e-4   ->  margin 2^-12 = 2.4e-4
+// so when the quick value lies farther than the margin from every integer, floor() of it IS the exact form's code.
+// The margin is added up front (so the test is one fract and one compare: fract(x + margin) >= 2 margin) and a value
+// that fails the test is requantised with the exact form.  About 2.4e-4 of the first-moment and 4.9e-4 of the
+// second-moment values of a continuous distribution fail it; values that sit on a rounding boundary to the last bit
+// (first steps from a zero state, sparse or lattice-valued gradients) always fail it.  The codes are therefore those
+// of the exact requantiser on any data, by construction; the stored scales are always formed from the correctly
+// rounded maximum.
+// Used by Adam on bf16 parameters with no or a 1-byte ECC (AdamQuickRequant); every other kernel evaluates the exact
+// forms only.
+constexpr float kQuickMarginMom = 0x1p-13f;
+constexpr float kQuickMarginVar = 0x1p-12f;
+// Quick pre-floor values (margin included).  rav255 = 255 * rcp(av), av = hw::sqrt of the group's largest v.
+FO_FN float quantize_mom_quick(float m, float am) {
+    const float t = m * hw::rcp(am + fabsf(m));  // = nm / (1 + |nm|), nm = m / am
+    return hw::fma(t, 254.0f, 0.5f + kQuickMarginMom);
+}
+FO_FN float quantize_var_quick(float r, float rav255) { return hw::fma(r, rav255, 0.5f + kQuickMarginVar); }
+// floor(x) is the exact form's code unless x (a quick value, margin included) lies within the margin of an integer.
+FO_FN bool quick_value_is_safe(float x, float margin) { return hw::fract(x) >= 2.0f * margin; }
+// One value through quick form, test and, if need be, exact form (what the kernels do, element by element).
+//   av_quick / av_exact: hw::sqrt and sqrt_corrected of the group's largest v; v: the element's second moment.
+FO_FN u32 quantize_mom_code_verified(float m, float am) {
+    const float x = quantize_mom_quick(m, am);
+    return quick_value_is_safe(x, kQuickMarginMom) ? (u32)hw::floor_to_int(x) : quantize_mom_code(m, am, hw::rcp(am));
+}
+FO_FN u32 quantize_var_code_verified(float v, float av_quick, float av_exact) {
+    const float x = quantize_var_quick(hw::sqrt(v), hw::rcp(av_quick) * 255.0f);
+    return quick_value_is_safe(x, kQuickMarginVar) ? (u32)(int)x : quantize_var_code(sqrt_corrected(v), av_exact, hw::rcp(av_exact));
+}
 
 // ------------------------------------------------------------------------------------------------
 // Adam / AdamW element update (ref:2296-2375)
@@ -321,11 +317,9 @@ template <int DT, int ECCB> struct AdamExact { static constexpr bool value = DT 
 // sit exactly on rounding boundaries in bulk, and the folded form's one-ulp differences then move up to 1e-2 of
 // the codes; with the unfolded moments and the exact requantiser their codes and scales equal the oracle's always.
 template <int DT, int ECCB> struct AdamFoldedMoments { static constexpr bool value = DT == DT_BF16; };
-// Variants whose wavefronts may take the quick requantiser: bf16 parameters with the folded update and no or a
-// 1-byte ECC.  Not with a 2-byte ECC, whose 14.25 bytes per element hide the exact requantiser's arithmetic
-// (measured: no gain).  Not fp16 parameters: their small gradients are fp16 subnormals, a handful of multiples of
-// 2^-24, and moments built from so few distinct values sit on rounding boundaries in bulk whatever the old state
-// is (measured: 1e-2 of the codes).
+// Variants that use the quick requantiser forms (verified element by element, see above): bf16 parameters with the
+// folded update and no or a 1-byte ECC.  With a 2-byte ECC the 14.25 bytes per element hide the exact
+// requantiser's arithmetic (measured: no gain); fp16 parameters are rare enough to keep the plain exact path.
 template <int DT, int ECCB> struct AdamQuickRequant { static constexpr bool value = DT == DT_BF16 && ECCB != 2; };
 
 // New moments from the dequantised pieces.

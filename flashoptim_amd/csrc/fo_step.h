@@ -87,29 +87,94 @@ __device__ __forceinline__ void write_master(const float (&p)[EPL], Pack<DTypeIn
 // Quantises the lane's first-moment values against the group absmax `am` (shared by the group's lanes, clamped
 // at 1e-12) and the lane's sqrt(v) values against the group maximum `av`; the rounding is the reference's
 // (fo_math.h: quantize_mom_rounded, quantize_var_rounded; ref:2405-2419, 1703-1710).
-template <int EPL, bool QUICK = false>
+template <int EPL>
 __device__ __forceinline__ void quantize_mom(const float (&m)[EPL], float am, Pack<1, EPL>& out) {
     static_assert(EPL == 8, "two dwords of codes per lane");
-    const float ram = QUICK ? 0.0f : hw::rcp(am);
+    const float ram = hw::rcp(am);
     float lo[4], hi[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        lo[k] = QUICK ? quantize_mom_quick(m[k], am) : quantize_mom_rounded(m[k], am, ram);
-        hi[k] = QUICK ? quantize_mom_quick(m[k + 4], am) : quantize_mom_rounded(m[k + 4], am, ram);
+        lo[k] = quantize_mom_rounded(m[k], am, ram);
+        hi[k] = quantize_mom_rounded(m[k + 4], am, ram);
     }
     convert_pack8<kFloor, kFloor>(lo, hi, out.w[0], out.w[1]);
 }
-template <int EPL, bool QUICK = false>
+template <int EPL>
 __device__ __forceinline__ void quantize_var(const float (&r)[EPL], float av, Pack<1, EPL>& out) {
     static_assert(EPL == 8, "two dwords of codes per lane");
-    const float rav = QUICK ? hw::rcp(av) * 255.0f : hw::rcp(av);
+    const float rav = hw::rcp(av);
     float lo[4], hi[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        lo[k] = QUICK ? quantize_var_quick(r[k], rav) : quantize_var_rounded(r[k], av, rav);
-        hi[k] = QUICK ? quantize_var_quick(r[k + 4], rav) : quantize_var_rounded(r[k + 4], av, rav);
+        lo[k] = quantize_var_rounded(r[k], av, rav);
+        hi[k] = quantize_var_rounded(r[k + 4], av, rav);
     }
     convert_pack8<kTrunc, kTrunc>(lo, hi, out.w[0], out.w[1]);
+}
+
+// Replaces byte k of the lane's eight packed codes.
+__device__ __forceinline__ void set_code(Pack<1, 8>& out, int k, u32 code) {
+    const int sh = 8 * (k & 3);
+    u32& w = out.w[k >> 2];
+    w = (w & ~(0xffu << sh)) | ((code & 0xffu) << sh);
+}
+
+// The same through the quick forms (fo_math.h): every value is converted from its quick form; the values that
+// fail the margin test are redone with the exact form.  A wavefront with no failing value (about four in five on
+// continuous data) branches past the repair; otherwise only the element positions k that failed in some lane are
+// redone.  The result is the exact requantiser's, code for code.
+template <int EPL>
+__device__ __forceinline__ void quantize_mom_quick_verified(const float (&m)[EPL], float am, Pack<1, EPL>& out) {
+    static_assert(EPL == 8, "two dwords of codes per lane");
+    float x[8];
+    bool redo[8];
+    bool any = false;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        x[k] = quantize_mom_quick(m[k], am);
+        redo[k] = !quick_value_is_safe(x[k], kQuickMarginMom);
+        any |= redo[k];
+    }
+    const float lo[4] = {x[0], x[1], x[2], x[3]}, hi[4] = {x[4], x[5], x[6], x[7]};
+    convert_pack8<kFloor, kFloor>(lo, hi, out.w[0], out.w[1]);
+    if (__builtin_amdgcn_ballot_w64(any) != 0) {
+        const float ram = hw::rcp(am);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            if (__builtin_amdgcn_ballot_w64(redo[k]) != 0) {
+                const u32 code = quantize_mom_code(m[k], am, ram);
+                if (redo[k]) set_code(out, k, code);
+            }
+        }
+    }
+}
+// r: hw::sqrt of the lane's second moments v; av_quick / av_exact: hw::sqrt and sqrt_corrected of the group's largest v.
+template <int EPL>
+__device__ __forceinline__ void quantize_var_quick_verified(const float (&v)[EPL], const float (&r)[EPL], float av_quick,
+                                                            float av_exact, Pack<1, EPL>& out) {
+    static_assert(EPL == 8, "two dwords of codes per lane");
+    const float rav255 = hw::rcp(av_quick) * 255.0f;
+    float x[8];
+    bool redo[8];
+    bool any = false;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        x[k] = quantize_var_quick(r[k], rav255);
+        redo[k] = !quick_value_is_safe(x[k], kQuickMarginVar);
+        any |= redo[k];
+    }
+    const float lo[4] = {x[0], x[1], x[2], x[3]}, hi[4] = {x[4], x[5], x[6], x[7]};
+    convert_pack8<kTrunc, kTrunc>(lo, hi, out.w[0], out.w[1]);
+    if (__builtin_amdgcn_ballot_w64(any) != 0) {
+        const float rav = hw::rcp(av_exact);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            if (__builtin_amdgcn_ballot_w64(redo[k]) != 0) {
+                const u32 code = quantize_var_code(sqrt_corrected(v[k]), av_exact, rav);
+                if (redo[k]) set_code(out, k, code);
+            }
+        }
+    }
 }
 // Four elements per lane (fp32 parameters): one dword of codes per state; the two states share the conversion block.
 __device__ __forceinline__ void quantize_mom_var(const float (&m)[4], float am, const float (&r)[4], float av,

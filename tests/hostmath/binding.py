@@ -43,6 +43,8 @@ def lib() -> ctypes.CDLL:
         L.hm_div_corrected.argtypes = [vp, vp, vp, i64]
         L.hm_sqrt_corrected.argtypes = [vp, vp, i64]
         L.hm_quantize_group.argtypes = [vp, vp, vp, vp, i64]
+        L.hm_quantize_group_from_moments.argtypes = [vp, vp, vp, vp, i64, i32]
+        L.hm_quantize_group_from_moments.restype = i64
         L.hm_ecc_join.argtypes = [vp, i32, vp, i32, vp, i64]
         L.hm_ecc_split.argtypes = [vp, vp, i32, vp, i32, i64, i32]
         L.hm_ecc_fraction_table.argtypes = [i32, vp, vp]
@@ -111,6 +113,16 @@ def quantize_group(m: torch.Tensor, r: torch.Tensor):
     qv = torch.empty(r.numel(), dtype=torch.uint8)
     lib().hm_quantize_group(_ptr(m), _ptr(r), _ptr(qm), _ptr(qv), m.numel())
     return qm, qv
+
+
+def quantize_group_from_moments(m: torch.Tensor, v: torch.Tensor, quick: bool):
+    """Codes of ONE group (all of m / v) from its moment values: through the quick forms with verification, or through
+    the exact forms alone.  Returns (first-moment codes, second-moment codes, number of values that failed the margin
+    test and were redone exactly)."""
+    qm = torch.empty(m.numel(), dtype=torch.int8)
+    qv = torch.empty(v.numel(), dtype=torch.uint8)
+    failed = lib().hm_quantize_group_from_moments(_ptr(m), _ptr(v), _ptr(qm), _ptr(qv), m.numel(), int(quick))
+    return qm, qv, int(failed)
 
 
 def ecc_join(narrow: torch.Tensor, ecc: torch.Tensor) -> torch.Tensor:

@@ -81,85 +81,65 @@ template <int DT, int ECCB> void write_master(void* param, void* ecc, int64_t i,
     if constexpr (ECCB > 0) store_ecc<ECCB>(ecc, i, ecc_split_bits<DT, ECCB, false>(p, w));
 }
 
-// the structure of adam_finish (fo_adam.hip), one wavefront span (64 lanes x EPL elements, counted from the start of
-// the tensor) at a time and one quantisation group at a time inside it: first the update of every group, with
-// sqrt(v) as the folded update takes it; then, like the kernel, the span-wide choice of the requantiser
-// (quick_requant_allowed for every group, else the exact forms on correctly rounded roots); then the codes.
+// the structure of adam_finish (fo_adam.hip), one quantisation group at a time
 template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT>
 void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scales, void* param, const void* grad, void* ecc,
                  int64_t n, const AdamHyper& h) {
-    constexpr int64_t kSpan = 64 * DTypeInfo<DT>::epl;
-    constexpr int kGroupsPerSpan = (int)(kSpan / kGroup);
-    constexpr bool kMayBeQuick = QUANT && !EXACT && AdamQuickRequant<DT, ECCB>::value;
-    struct GroupWork { float m[kGroup], r[kGroup], v[kGroup], am, av, gmax; int cnt; };
-    static thread_local GroupWork work[kGroupsPerSpan];
-    for (int64_t s0 = 0; s0 < n; s0 += kSpan) {
-        const int64_t s1 = (s0 + kSpan) < n ? (s0 + kSpan) : n;
-        bool quick = kMayBeQuick;
-        int n_groups = 0;
-        for (int64_t g0 = s0; g0 < s1; g0 += kGroup, ++n_groups) {
-            GroupWork& w = work[n_groups];
-            w.cnt = (int)((n - g0) < kGroup ? (n - g0) : kGroup);
-            const int64_t group = g0 >> 5;
-            float sm = 1.0f, sv = 1.0f;
-            if (QUANT) { sm = f16_to_f32(mom_scales[group]); sv = f16_to_f32(var_scales[group]); }
-            const float sm_b1 = sm * h.b1, sv_b2 = sv * h.sqrt_b2_over_255;
-            w.am = 0.0f; w.av = 0.0f; w.gmax = 0.0f;
-            for (int k = 0; k < w.cnt; ++k) {
-                const int64_t i = g0 + k;
-                float p = read_master<DT, ECCB>(param, ecc, i);
-                float gr = load_elem<DT>(grad, i);
-                if (!DECOUPLED) gr = gr + p * h.wd;
-                w.gmax = fmaxf(w.gmax, fabsf(gr));
-                float mn, vn;
-                if (QUANT) {
-                    adam_moments_quantized<(EXACT || !AdamFoldedMoments<DT, ECCB>::value)>(gr, kTable.v[((const uint8_t*)mom)[i]], sm, sm_b1,
-                                                  (float)((const uint8_t*)var)[i], sv, sv_b2, h, mn, vn);
-                } else {
-                    adam_moments_plain(gr, load_elem<DT>(mom, i), load_elem<DT>(var, i), h, mn, vn);
-                }
-                if (DECOUPLED) p = p * h.one_m_wd;
-                const float rk = (QUANT || !EXACT) ? (kMayBeQuick ? hw::sqrt(vn) : sqrt_corrected(vn)) : 0.0f;
-                p = adam_apply<EXACT>(p, mn, vn, rk, h);
-                write_master<DT, ECCB>(param, ecc, i, p);
-                w.m[k] = mn; w.r[k] = rk; w.v[k] = vn;
-                w.am = fmaxf(w.am, fabsf(mn));
-                w.av = fmaxf(w.av, rk);
+    constexpr bool kQuick = QUANT && !EXACT && AdamQuickRequant<DT, ECCB>::value;
+    constexpr bool kExactMoments = EXACT || !AdamFoldedMoments<DT, ECCB>::value;
+    for (int64_t g0 = 0; g0 < n; g0 += kGroup) {
+        const int cnt = (int)((n - g0) < kGroup ? (n - g0) : kGroup);
+        const int64_t group = g0 >> 5;
+        float sm = 1.0f, sv = 1.0f;
+        if (QUANT) { sm = f16_to_f32(mom_scales[group]); sv = f16_to_f32(var_scales[group]); }
+        const float sm_b1 = sm * h.b1, sv_b2 = sv * h.sqrt_b2_over_255;
+        float m[kGroup], r[kGroup], v[kGroup];
+        float am = 0.0f, av = 0.0f, vmax = 0.0f;
+        for (int k = 0; k < cnt; ++k) {
+            const int64_t i = g0 + k;
+            float p = read_master<DT, ECCB>(param, ecc, i);
+            float gr = load_elem<DT>(grad, i);
+            if (!DECOUPLED) gr = gr + p * h.wd;
+            float mn, vn;
+            if (QUANT) {
+                adam_moments_quantized<kExactMoments>(gr, kTable.v[((const uint8_t*)mom)[i]], sm, sm_b1,
+                                                      (float)((const uint8_t*)var)[i], sv, sv_b2, h, mn, vn);
+            } else {
+                adam_moments_plain(gr, load_elem<DT>(mom, i), load_elem<DT>(var, i), h, mn, vn);
             }
-            if (kMayBeQuick && !quick_requant_allowed(mom_scales[group], var_scales[group], sm_b1, w.am, sv_b2, w.av, w.gmax,
-                                                       h.one_m_b1, h.one_m_b2))
-                quick = false;
-            w.am = fmaxf(w.am, 1e-12f);
+            if (DECOUPLED) p = p * h.one_m_wd;
+            const float rk = (QUANT || !EXACT) ? (kQuick ? hw::sqrt(vn) : sqrt_corrected(vn)) : 0.0f;
+            p = adam_apply<EXACT>(p, mn, vn, rk, h);
+            write_master<DT, ECCB>(param, ecc, i, p);
+            m[k] = mn; r[k] = rk; v[k] = vn;
+            am = fmaxf(am, fabsf(mn));
+            av = fmaxf(av, rk);
+            vmax = fmaxf(vmax, vn);
         }
-        int gi = 0;
-        for (int64_t g0 = s0; g0 < s1; g0 += kGroup, ++gi) {
-            GroupWork& w = work[gi];
-            const int64_t group = g0 >> 5;
-            if (!QUANT) {
-                for (int k = 0; k < w.cnt; ++k) {
-                    store_elem<DT>(mom, g0 + k, w.m[k]);
-                    store_elem<DT>(var, g0 + k, w.v[k]);
+        if (QUANT) {
+            am = fmaxf(am, 1e-12f);
+            if (kQuick) {  // quick forms, each value verified and redone exactly if it fails (fo_math.h)
+                const float av_quick = fmaxf(hw::sqrt(vmax), 1e-12f);
+                av = fmaxf(sqrt_corrected(vmax), 1e-12f);
+                for (int k = 0; k < cnt; ++k) {
+                    ((uint8_t*)mom)[g0 + k] = (uint8_t)quantize_mom_code_verified(m[k], am);
+                    ((uint8_t*)var)[g0 + k] = (uint8_t)quantize_var_code_verified(v[k], av_quick, av);
                 }
-                continue;
-            }
-            if (kMayBeQuick && !quick) {  // the exact requantiser wants the correctly rounded roots and their maximum
-                w.av = 0.0f;
-                for (int k = 0; k < w.cnt; ++k) { w.r[k] = sqrt_corrected(w.v[k]); w.av = fmaxf(w.av, w.r[k]); }
-            }
-            w.av = fmaxf(w.av, 1e-12f);
-            const float ram = hw::rcp(w.am), rav = hw::rcp(w.av);
-            const float rav255 = rav * 255.0f;
-            for (int k = 0; k < w.cnt; ++k) {
-                if (kMayBeQuick && quick) {
-                    ((uint8_t*)mom)[g0 + k] = (uint8_t)hw::floor_to_int(quantize_mom_quick(w.m[k], w.am));
-                    ((uint8_t*)var)[g0 + k] = (uint8_t)(int)quantize_var_quick(w.r[k], rav255);
-                } else {
-                    ((uint8_t*)mom)[g0 + k] = (uint8_t)quantize_mom_code(w.m[k], w.am, ram);
-                    ((uint8_t*)var)[g0 + k] = (uint8_t)quantize_var_code(w.r[k], w.av, rav);
+            } else {
+                av = fmaxf(av, 1e-12f);
+                const float ram = hw::rcp(am), rav = hw::rcp(av);
+                for (int k = 0; k < cnt; ++k) {
+                    ((uint8_t*)mom)[g0 + k] = (uint8_t)quantize_mom_code(m[k], am, ram);
+                    ((uint8_t*)var)[g0 + k] = (uint8_t)quantize_var_code(r[k], av, rav);
                 }
             }
-            mom_scales[group] = f32_to_f16(w.am);
-            var_scales[group] = f32_to_f16(w.av);
+            mom_scales[group] = f32_to_f16(am);
+            var_scales[group] = f32_to_f16(av);
+        } else {
+            for (int k = 0; k < cnt; ++k) {
+                store_elem<DT>(mom, g0 + k, m[k]);
+                store_elem<DT>(var, g0 + k, v[k]);
+            }
         }
     }
 }
@@ -280,6 +260,28 @@ void hm_ecc_fraction_table(int dtype, float* table_out, float* arithmetic_out) {
         if (dtype == DT_BF16) { table_out[b] = kTables<DT_BF16>.v[256 + b]; arithmetic_out[b] = ecc_fraction<DT_BF16, 1>(q); }
         else { table_out[b] = kTables<DT_F16>.v[256 + b]; arithmetic_out[b] = ecc_fraction<DT_F16, 1>(q); }
     }
+}
+// codes of one group from its first-moment values m and second-moment values v: through the quick forms with
+// verification (quick != 0) or through the exact forms alone; also how many values failed the margin test
+int64_t hm_quantize_group_from_moments(const float* m, const float* v, int8_t* qm, uint8_t* qv, int64_t n, int quick) {
+    float am = 0.0f, vmax = 0.0f;
+    for (int64_t i = 0; i < n; ++i) { am = fmaxf(am, fabsf(m[i])); vmax = fmaxf(vmax, v[i]); }
+    am = fmaxf(am, 1e-12f);
+    const float av_quick = fmaxf(hw::sqrt(vmax), 1e-12f), av = fmaxf(sqrt_corrected(vmax), 1e-12f);
+    const float ram = hw::rcp(am), rav = hw::rcp(av);
+    int64_t failed = 0;
+    for (int64_t i = 0; i < n; ++i) {
+        if (quick) {
+            qm[i] = (int8_t)quantize_mom_code_verified(m[i], am);
+            qv[i] = (uint8_t)quantize_var_code_verified(v[i], av_quick, av);
+            failed += !quick_value_is_safe(quantize_mom_quick(m[i], am), kQuickMarginMom);
+            failed += !quick_value_is_safe(quantize_var_quick(hw::sqrt(v[i]), hw::rcp(av_quick) * 255.0f), kQuickMarginVar);
+        } else {
+            qm[i] = (int8_t)quantize_mom_code(m[i], am, ram);
+            qv[i] = (uint8_t)quantize_var_code(sqrt_corrected(v[i]), av, rav);
+        }
+    }
+    return failed;
 }
 void hm_softsign_table(float* out) { for (int b = 0; b < 256; ++b) out[b] = kTable.v[b]; }
 

@@ -7,11 +7,11 @@ identical inputs:
 * Adam with fp16 parameters (folded update, unfolded moments): codes and scales bit-exact, master weights and
   narrow parameters as in the next item;
 * Adam with bf16 parameters (folded update and moments): the new moments come out of fused multiply-adds and may
-  differ from the oracle's by an ulp, and wavefront spans in which every group's new maxima carry old state
-  requantise with the quick forms (a few ulps off; no or 1-byte ECC only), so
+  differ from the oracle's by an ulp (the requantiser itself yields the exact forms' codes: its quick forms are
+  verified value by value), so
   - 8-bit moment codes never differ by more than +-1 code step and differ on fewer than 0.01 % of the elements
     (measured 1e-6 .. 2.5e-5; exactly 0 on a first step from zero states and in any group that starts from zero,
-    where m and v are formed identically and the exact requantiser runs);
+    where m and v are formed identically);
   - fp16 group scales: equal, or one fp16 ulp apart on fewer than 0.1 % of the groups;
   - master weights (narrow parameter + ECC): within one unit of master precision, i.e. half-ulp(narrow)/127 for
     24-bit, /32767 for 32-bit masters; plus one fp32 ulp (the updated value is rounded to fp32 before it is

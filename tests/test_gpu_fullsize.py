@@ -1,9 +1,7 @@
 """Full-size checks of the step kernels through properties that do not need the oracle at that size.
 
 The update is elementwise and every 32-element group is independent, so the step on any group-aligned window of a
-tensor must equal, bit for bit, the same kernel run on a copy of that window alone (the Adam kernels on 2-byte
-parameters choose between two requantisers per 512-element span counted from the start of the tensor; the states
-here are zero or warm throughout, so every span chooses alike wherever it starts).  Windows are sampled across a
+tensor must equal, bit for bit, the same kernel run on a copy of that window alone.  Windows are sampled across a
 2^30-element tensor (the flat throughput configuration) and across a tensor longer than 2^31 elements (beyond the
 reference's int32 indexing; byte offsets pass 2^32), including the ragged tail, and a few of them are also checked
 against the CPU oracle with the usual parity tolerances.  Together with the small-size oracle parity this pins the

@@ -250,8 +250,9 @@ def test_adam_headline_config_code_mismatch_rate(ecc_dtype):
 @pytest.mark.parametrize("dtype,ecc_dtype", [(torch.bfloat16, torch.int8), (torch.float16, torch.int8), (torch.bfloat16, None), (torch.bfloat16, torch.int16)])
 def test_adam_groups_that_start_from_zero_get_the_exact_requantiser(dtype, ecc_dtype):
     """Two steps, then 2 % of the groups are reset to a zero state (as if they had seen no gradient yet) and a
-    third step is taken: every code of a reset group equals the oracle's, whichever requantiser the rest of its
-    wavefront span would have taken; all other codes meet the usual rate."""
+    third step is taken: every code of a reset group equals the oracle's (their values sit on rounding boundaries in
+    bulk; the quick requantiser forms must hand every such value to the exact form); all other codes meet the usual
+    rate."""
     k = _k()
     n = (1 << 17) + 17
     c = _Case(n, dtype, ecc_dtype, True, 2, seed=5)
@@ -278,8 +279,8 @@ def test_adam_groups_that_start_from_zero_get_the_exact_requantiser(dtype, ecc_d
 
 def test_adam_sudden_jump_of_the_gradient_scale_keeps_the_code_tolerance():
     """Three steps at gradient scale 1e-4, then one step with gradients 1 to 1e5 times larger: the old second moment
-    becomes negligible, the new values sit near rounding boundaries as on a first step, and the kernel must fall
-    back to the exact requantiser for such groups (quick forms alone: up to 0.4 % of the codes off)."""
+    becomes negligible, the new values sit near rounding boundaries as on a first step, and the margin test of the
+    quick requantiser forms must hand them to the exact form (quick forms alone: up to 0.4 % of the codes off)."""
     k = _k()
     n = (1 << 18) + 5
     lr, b1, b2, eps, wd = 1e-3, 0.9, 0.999, 1e-8, 1e-5
@@ -299,8 +300,7 @@ def test_adam_sudden_jump_of_the_gradient_scale_keeps_the_code_tolerance():
 
 @pytest.mark.parametrize("betas", [(0.0, 0.999), (0.9, 0.0), (0.0, 0.0), (0.01, 0.999), (0.9, 0.1), (0.5, 0.9), (0.99, 0.9999)])
 def test_adam_code_tolerance_holds_for_unusual_betas(betas):
-    """beta1 = 0 or beta2 = 0: the old state has no weight and every step is as tie-prone as a first step; the
-    kernel must keep such steps on the exact requantiser."""
+    """beta1 = 0 or beta2 = 0: the old state has no weight and every step is as tie-prone as a first step."""
     k = _k()
     n = (1 << 18) + 5
     c = _Case(n, torch.bfloat16, torch.int8, True, 2, seed=3)
@@ -553,7 +553,7 @@ def test_step_kernels_are_resident_as_planned():
     import ctypes
 
     lib = _native_lib()
-    want_adam = {(0, 0): 20, (1, 0): 15, (1, 1): 15, (1, 2): 16, (2, 0): 15, (2, 1): 15, (2, 2): 16}
+    want_adam = {(0, 0): 20, (1, 0): 16, (1, 1): 16, (1, 2): 16, (2, 0): 16, (2, 1): 16, (2, 2): 16}
     for (dtype, ecc), want in want_adam.items():
         for quantized in (1, 0):
             for multi in (0, 1):
