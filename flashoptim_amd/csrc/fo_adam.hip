@@ -42,7 +42,8 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
     constexpr int EPL = DTypeInfo<DT>::epl;
     constexpr int PB = DTypeInfo<DT>::bytes;
     constexpr int SB = QUANT ? 1 : PB;
-    constexpr bool MAY_BE_QUICK = QUANT && !EXACT && AdamQuickRequant<DT, ECCB>::value;  // fo_math.h: "two requantisers"
+    // the requantiser goes through the quick forms, every value verified (fo_math.h)
+    constexpr bool MAY_BE_QUICK = QUANT && AdamQuickRequant<DT, ECCB>::value && (!EXACT || AdamExact<DT, ECCB>::value);
     constexpr bool EXACT_MOMENTS = EXACT || !AdamFoldedMoments<DT, ECCB>::value;
     const int64_t n = t.n;
     const bool live_group = FAST == kVector || w.first() < n;  // the lane owns at least one real element
@@ -89,11 +90,14 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
         am = fmaxf(group_max<EPL>(am), 1e-12f);
         av = group_max<EPL>(av);
         if constexpr (MAY_BE_QUICK) {
-            static_assert(EPL == 8, "2-byte parameters");
             const float av_quick = fmaxf(hw::sqrt(av), 1e-12f);   // av holds the group's largest v here
             av = fmaxf(sqrt_corrected(av), 1e-12f);               // what the exact requantiser divides by, and the scale
-            quantize_mom_quick_verified<EPL>(m, am, raw.m);
-            quantize_var_quick_verified<EPL>(v, r, av_quick, av, raw.v);
+            if constexpr (EPL == 8) {
+                quantize_mom_quick_verified<EPL>(m, am, raw.m);
+                quantize_var_quick_verified<EPL>(v, r, av_quick, av, raw.v);
+            } else {
+                quantize_mom_var_quick_verified(m, am, v, r, av_quick, av, raw.m, raw.v);
+            }
         } else if constexpr (EPL == 8) {
             av = fmaxf(av, 1e-12f);
             quantize_mom<EPL>(m, am, raw.m);

@@ -317,10 +317,11 @@ template <int DT, int ECCB> struct AdamExact { static constexpr bool value = DT 
 // sit exactly on rounding boundaries in bulk, and the folded form's one-ulp differences then move up to 1e-2 of
 // the codes; with the unfolded moments and the exact requantiser their codes and scales equal the oracle's always.
 template <int DT, int ECCB> struct AdamFoldedMoments { static constexpr bool value = DT == DT_BF16; };
-// Variants that use the quick requantiser forms (verified element by element, see above): bf16 parameters with the
-// folded update and no or a 1-byte ECC.  With a 2-byte ECC the 14.25 bytes per element hide the exact
-// requantiser's arithmetic (measured: no gain); fp16 parameters are rare enough to keep the plain exact path.
-template <int DT, int ECCB> struct AdamQuickRequant { static constexpr bool value = DT == DT_BF16 && ECCB != 2; };
+// Variants that use the quick requantiser forms (verified value by value, see above; the codes are the exact
+// forms' either way): bf16 parameters with no or a 1-byte ECC, and fp32 parameters.  With a 2-byte ECC the
+// 14.25 bytes per element hide the exact requantiser's arithmetic (measured: no gain); fp16 parameters and the
+// operation-by-operation update on 2-byte parameters are rare enough to keep the plain exact path.
+template <int DT, int ECCB> struct AdamQuickRequant { static constexpr bool value = (DT == DT_BF16 && ECCB != 2) || DT == DT_F32; };
 
 // New moments from the dequantised pieces.
 //   EXACT = false: the EMA decay is folded into the group scale (one multiply per lane instead of one per

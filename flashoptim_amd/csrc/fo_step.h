@@ -112,8 +112,8 @@ __device__ __forceinline__ void quantize_var(const float (&r)[EPL], float av, Pa
     convert_pack8<kTrunc, kTrunc>(lo, hi, out.w[0], out.w[1]);
 }
 
-// Replaces byte k of the lane's eight packed codes.
-__device__ __forceinline__ void set_code(Pack<1, 8>& out, int k, u32 code) {
+// Replaces byte k of the lane's packed codes.
+template <int EPL> __device__ __forceinline__ void set_code(Pack<1, EPL>& out, int k, u32 code) {
     const int sh = 8 * (k & 3);
     u32& w = out.w[k >> 2];
     w = (w & ~(0xffu << sh)) | ((code & 0xffu) << sh);
@@ -143,7 +143,7 @@ __device__ __forceinline__ void quantize_mom_quick_verified(const float (&m)[EPL
         for (int k = 0; k < 8; ++k) {
             if (__builtin_amdgcn_ballot_w64(redo[k]) != 0) {
                 const u32 code = quantize_mom_code(m[k], am, ram);
-                if (redo[k]) set_code(out, k, code);
+                if (redo[k]) set_code<EPL>(out, k, code);
             }
         }
     }
@@ -171,7 +171,40 @@ __device__ __forceinline__ void quantize_var_quick_verified(const float (&v)[EPL
         for (int k = 0; k < 8; ++k) {
             if (__builtin_amdgcn_ballot_w64(redo[k]) != 0) {
                 const u32 code = quantize_var_code(sqrt_corrected(v[k]), av_exact, rav);
-                if (redo[k]) set_code(out, k, code);
+                if (redo[k]) set_code<EPL>(out, k, code);
+            }
+        }
+    }
+}
+// Four elements per lane (fp32 parameters), both states through the quick forms with verification: one conversion
+// block, one repair branch.
+__device__ __forceinline__ void quantize_mom_var_quick_verified(const float (&m)[4], float am, const float (&v)[4],
+                                                                const float (&r)[4], float av_quick, float av_exact,
+                                                                Pack<1, 4>& mout, Pack<1, 4>& vout) {
+    const float rav255 = hw::rcp(av_quick) * 255.0f;
+    float xm[4], xv[4];
+    bool redo_m[4], redo_v[4];
+    bool any = false;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        xm[k] = quantize_mom_quick(m[k], am);
+        xv[k] = quantize_var_quick(r[k], rav255);
+        redo_m[k] = !quick_value_is_safe(xm[k], kQuickMarginMom);
+        redo_v[k] = !quick_value_is_safe(xv[k], kQuickMarginVar);
+        any |= redo_m[k] | redo_v[k];
+    }
+    convert_pack8<kFloor, kTrunc>(xm, xv, mout.w[0], vout.w[0]);
+    if (__builtin_amdgcn_ballot_w64(any) != 0) {
+        const float ram = hw::rcp(am), rav = hw::rcp(av_exact);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if (__builtin_amdgcn_ballot_w64(redo_m[k]) != 0) {
+                const u32 code = quantize_mom_code(m[k], am, ram);
+                if (redo_m[k]) set_code<4>(mout, k, code);
+            }
+            if (__builtin_amdgcn_ballot_w64(redo_v[k]) != 0) {
+                const u32 code = quantize_var_code(sqrt_corrected(v[k]), av_exact, rav);
+                if (redo_v[k]) set_code<4>(vout, k, code);
             }
         }
     }
