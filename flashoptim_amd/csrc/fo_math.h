@@ -242,8 +242,8 @@ FO_FN u32 quantize_var_code(float r, float av, float rav) { return (u32)(int)qua
 // (first steps from a zero state, sparse or lattice-valued gradients) always fail it.  The codes are therefore those
 // of the exact requantiser on any data, by construction; the stored scales are always formed from the correctly
 // rounded maximum.
-// Used by Adam on bf16 parameters with no or a 1-byte ECC (AdamQuickRequant); every other kernel evaluates the exact
-// forms only.
+// Used by Adam on bf16 parameters with no or a 1-byte ECC and on fp32 parameters (AdamQuickRequant) and by the
+// momentum kernels on 2-byte parameters; the other kernels evaluate the exact forms only.
 constexpr float kQuickMarginMom = 0x1p-13f;
 constexpr float kQuickMarginVar = 0x1p-12f;
 // Quick pre-floor values (margin included).  rav255 = 255 * rcp(av), av = hw::sqrt of the group's largest v.

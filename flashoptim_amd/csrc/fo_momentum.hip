@@ -71,7 +71,9 @@ __device__ __forceinline__ void momentum_finish(const TensorPtrs& t, Where w, Mo
     if constexpr (KIND != KIND_PLAIN) {
         if constexpr (QUANT) {
             am = fmaxf(group_max<EPL>(am), 1e-12f);                                 // ref:1702-1703
-            quantize_mom(m, am, raw.m);
+            // 2-byte parameters: through the quick forms, every value verified (fo_math.h): the exact forms' codes
+            if constexpr (EPL == 8) quantize_mom_quick_verified<EPL>(m, am, raw.m);
+            else quantize_mom(m, am, raw.m);
             store_lane<1, EPL, FAST>(raw.m, t.mom, w, n);
             if (live_group && (threadIdx.x & (32 / EPL - 1)) == 0) store_scale(t.mom_scales, w, f32_to_f16_bits(am));  // ref:1713-1716
         } else {

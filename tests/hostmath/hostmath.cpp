@@ -168,7 +168,8 @@ void momentum_tensor(void* mom, uint16_t* mom_scales, void* param, const void* g
         if (QUANT) {
             am = fmaxf(am, 1e-12f);
             const float ram = hw::rcp(am);
-            for (int k = 0; k < cnt; ++k) ((uint8_t*)mom)[g0 + k] = (uint8_t)quantize_mom_code(m[k], am, ram);
+            for (int k = 0; k < cnt; ++k)  // as momentum_finish: 2-byte parameters go through the verified quick forms
+                ((uint8_t*)mom)[g0 + k] = (uint8_t)(DT == DT_F32 ? quantize_mom_code(m[k], am, ram) : quantize_mom_code_verified(m[k], am));
             mom_scales[group] = f32_to_f16(am);
         } else {
             for (int k = 0; k < cnt; ++k) store_elem<DT>(mom, g0 + k, m[k]);
