@@ -43,7 +43,7 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
     constexpr int PB = DTypeInfo<DT>::bytes;
     constexpr int SB = QUANT ? 1 : PB;
     // the requantiser goes through the quick forms, every value verified (fo_math.h)
-    constexpr bool MAY_BE_QUICK = QUANT && AdamQuickRequant<DT, ECCB>::value && (!EXACT || AdamExact<DT, ECCB>::value);
+    constexpr bool MAY_BE_QUICK = QUANT && (AdamQuickRequant<DT, ECCB>::value || EXACT);
     constexpr bool EXACT_MOMENTS = EXACT || !AdamFoldedMoments<DT, ECCB>::value;
     const int64_t n = t.n;
     const bool live_group = FAST == kVector || w.first() < n;  // the lane owns at least one real element
@@ -129,9 +129,8 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT = AdamExact<D
     // measured on MI355X with the 8B-parameter step and this file's ILP-oriented instruction schedule: 16-17
     // resident workgroups per compute unit for 2-byte parameters (3.6-4.6 KiB of loads per wavefront; 15 and 18
     // are two to three points worse on the 8B list, a flat tensor does not care between 15 and 17), 18-20 for fp32
-    // parameters (2.5 KiB).  The operation-by-operation update on 2-byte parameters is arithmetic-bound and gets
-    // what its 90-99 VGPRs allow.
-    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 20 : 16;
+    // parameters (2.5 KiB) and for the arithmetic-bound operation-by-operation update on 2-byte parameters.
+    static constexpr int kWorkgroupsPerCu = (DT == DT_F32 || EXACT) ? 20 : 16;
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {

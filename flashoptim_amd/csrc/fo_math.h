@@ -242,8 +242,8 @@ FO_FN u32 quantize_var_code(float r, float av, float rav) { return (u32)(int)qua
 // (first steps from a zero state, sparse or lattice-valued gradients) always fail it.  The codes are therefore those
 // of the exact requantiser on any data, by construction; the stored scales are always formed from the correctly
 // rounded maximum.
-// Used by Adam on bf16 parameters with no or a 1-byte ECC and on fp32 parameters (AdamQuickRequant) and by the
-// momentum kernels on 2-byte parameters; the other kernels evaluate the exact forms only.
+// Used by the Adam kernels (all but the folded update with a 2-byte ECC, AdamQuickRequant) and by the momentum
+// kernels on 2-byte parameters; the other kernels evaluate the exact forms only.
 constexpr float kQuickMarginMom = 0x1p-13f;
 constexpr float kQuickMarginVar = 0x1p-12f;
 // Quick pre-floor values (margin included).  rav255 = 255 * rcp(av), av = hw::sqrt of the group's largest v.
@@ -318,10 +318,9 @@ template <int DT, int ECCB> struct AdamExact { static constexpr bool value = DT 
 // the codes; with the unfolded moments and the exact requantiser their codes and scales equal the oracle's always.
 template <int DT, int ECCB> struct AdamFoldedMoments { static constexpr bool value = DT == DT_BF16; };
 // Variants that use the quick requantiser forms (verified value by value, see above; the codes are the exact
-// forms' either way): bf16 parameters with no or a 1-byte ECC, and fp32 parameters.  With a 2-byte ECC the
-// 14.25 bytes per element hide the exact requantiser's arithmetic (measured: no gain); fp16 parameters and the
-// operation-by-operation update on 2-byte parameters are rare enough to keep the plain exact path.
-template <int DT, int ECCB> struct AdamQuickRequant { static constexpr bool value = (DT == DT_BF16 && ECCB != 2) || DT == DT_F32; };
+// forms' either way): all but the folded update with a 2-byte ECC, whose 14.25 bytes per element hide the exact
+// requantiser's arithmetic (measured: no gain).  The operation-by-operation update uses them with any ECC width.
+template <int DT, int ECCB> struct AdamQuickRequant { static constexpr bool value = DT == DT_F32 || ECCB != 2; };
 
 // New moments from the dequantised pieces.
 //   EXACT = false: the EMA decay is folded into the group scale (one multiply per lane instead of one per

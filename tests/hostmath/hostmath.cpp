@@ -85,7 +85,7 @@ template <int DT, int ECCB> void write_master(void* param, void* ecc, int64_t i,
 template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT>
 void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scales, void* param, const void* grad, void* ecc,
                  int64_t n, const AdamHyper& h) {
-    constexpr bool kQuick = QUANT && AdamQuickRequant<DT, ECCB>::value && (!EXACT || AdamExact<DT, ECCB>::value);
+    constexpr bool kQuick = QUANT && (AdamQuickRequant<DT, ECCB>::value || EXACT);
     constexpr bool kExactMoments = EXACT || !AdamFoldedMoments<DT, ECCB>::value;
     for (int64_t g0 = 0; g0 < n; g0 += kGroup) {
         const int cnt = (int)((n - g0) < kGroup ? (n - g0) : kGroup);
