@@ -142,6 +142,45 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT = AdamExact<D
     }
 };
 
+
+// The Adam step's memory accesses without its arithmetic: every stream of the step is loaded and stored back
+// unchanged through the same load / store code, launch geometry and residency mechanism.  It shows what rate this
+// mix of seven loads and six stores per wavefront reaches on the device, next to the step kernels' own rate.
+// `mask` arrives as zero from the entry point; folding the gradient words in under it keeps the gradient loads
+// alive without changing any byte.
+struct StreamsHyper { uint32_t mask; };
+
+template <int DT, int ECCB, bool QUANT> struct AdamStreamsOp {
+    using Hyper = StreamsHyper;
+    static constexpr int kLutTables = 0;
+    static constexpr int kDtype = DT;
+    // where this copy streams fastest on MI355X with the 8B-parameter list: 16-17 with 1-byte ECC (14-15 and 18-20
+    // are three to four points slower), 14-15 with 2-byte ECC (16-17 one point slower)
+    static constexpr int kWorkgroupsPerCu = ECCB == 2 ? 15 : 16;
+    static constexpr int kEpl = DTypeInfo<DT>::epl;
+    using Raw = AdamRaw<DT, ECCB, QUANT>;
+    template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {
+        adam_load<DT, ECCB, QUANT, FAST>(t, w, r);
+    }
+    template <int FAST>
+    __device__ __forceinline__ static void finish(const TensorPtrs& t, Where w, Raw& r, const Hyper& h, const float*) {
+        constexpr int PB = DTypeInfo<DT>::bytes;
+        constexpr int SB = QUANT ? 1 : PB;
+#pragma unroll
+        for (int i = 0; i < Pack<PB, kEpl>::kDwords; ++i) r.p.w[i] ^= r.g.w[i] & h.mask;
+        store_lane<PB, kEpl, FAST>(r.p, t.param, w, t.n);
+        store_lane<ECCB, kEpl, FAST>(r.e, t.ecc, w, t.n);
+        store_lane<SB, kEpl, FAST>(r.m, t.mom, w, t.n);
+        store_lane<SB, kEpl, FAST>(r.v, t.var, w, t.n);
+        if constexpr (QUANT) {
+            if ((FAST == kVector || w.first() < t.n) && (threadIdx.x & (32 / kEpl - 1)) == 0) {
+                store_scale(t.mom_scales, w, r.sm);
+                store_scale(t.var_scales, w, r.sv);
+            }
+        }
+    }
+};
+
 }  // namespace fo
 
 namespace {
@@ -335,6 +374,14 @@ int fo_multi_adam_step_static(const fo_tensor_desc* host_descs, int64_t n_tensor
     }
     MultiLauncher<fo::AdamHyper> L{d_descs, d_chunks, n_chunks, make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step), (hipStream_t)stream};
     return decoupled ? dispatch<AdamWOp>(dtype, ecc_bytes, quantized, L) : dispatch<AdamL2Op>(dtype, ecc_bytes, quantized, L);
+}
+
+int fo_multi_adam_streams_copy(const fo_tensor_desc* descs, int64_t n_tensors, const fo_chunk* chunks, int64_t n_chunks,
+                               int dtype, int ecc_bytes, int quantized, void* stream) {
+    if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
+    if (n_chunks == 0) return 0;
+    MultiLauncher<fo::StreamsHyper> L{descs, chunks, n_chunks, fo::StreamsHyper{0u}, (hipStream_t)stream};
+    return dispatch<fo::AdamStreamsOp>(dtype, ecc_bytes, quantized, L);
 }
 
 int fo_adam_step_residency(int dtype, int ecc_bytes, int quantized, int decoupled, int multi, int* target, int* achieved,

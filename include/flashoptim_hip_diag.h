@@ -9,6 +9,8 @@
 
 #include <stdint.h>
 
+#include "flashoptim_hip.h"
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -19,6 +21,16 @@ extern "C" {
  * kernels.  n_bytes must be a multiple of 16 and both pointers 16-byte aligned.
  */
 int fo_copy_bytes(void *dst, const void *src, int64_t n_bytes, void *stream);
+
+/*
+ * The Adam step's memory accesses without its arithmetic: every tensor of the table is read (parameters, gradients,
+ * ECC, both moments and their group scales) and written back unchanged (everything but the gradients) by the step
+ * kernels' own load / store code, launch geometry and residency mechanism.  Arguments as fo_multi_adam_step's
+ * (flashoptim_hip.h) without the scalars.  The rate it reaches is the ceiling of the step's access mix on the
+ * device, to be read next to the step's own rate and to fo_copy_bytes' (one load and one store stream).
+ */
+int fo_multi_adam_streams_copy(const fo_tensor_desc *descs, int64_t n_tensors, const fo_chunk *chunks, int64_t n_chunks,
+                               int dtype, int ecc_bytes, int quantized, void *stream);
 
 /*
  * Residency plan of a step kernel on the current device: the workgroups per compute unit the kernel family asks

@@ -495,6 +495,40 @@ def test_kernels_never_write_outside_their_tensors(n):
             assert bool(torch.isfinite(f["p"].t.float()).all())
 
 
+@pytest.mark.parametrize("n", [1, 33, 511, 4096, 4097, 3 * 4096 + 40, 1 << 20])
+def test_access_mix_copy_changes_no_byte(n):
+    """The measurement kernel that runs the Adam step's loads and stores without its arithmetic leaves parameters,
+    gradients, ECC, codes and scales exactly as they were, and the bytes next to them untouched (bf16 with both ECC
+    widths, fp16, fp32; two tensors per launch, one of them after a real step so that no stream is all zero)."""
+    k = _k()
+    from flashoptim_amd.launcher import BucketPlan, StepTensors
+
+    groups = (n + 31) // 32
+    for dtype, ecc_dtype in ((torch.bfloat16, torch.int8), (torch.bfloat16, torch.int16), (torch.float16, torch.int8),
+                             (torch.float32, None)):
+        def fenced_set(seed):
+            f = dict(p=_Fenced(n, dtype), g=_Fenced(n, dtype), m=_Fenced(n, torch.int8), ms=_Fenced(groups, torch.float16),
+                     v=_Fenced(n, torch.uint8), vs=_Fenced(groups, torch.float16))
+            f["p"].t.copy_(_rand(n, 0.02, seed).to(dtype))
+            f["g"].t.copy_(_rand(n, 1e-3, seed + 1).to(dtype))
+            f["e"] = None if ecc_dtype is None else _Fenced(n, ecc_dtype)
+            return f
+
+        a, b = fenced_set(1), fenced_set(3)
+        ecc = lambda f: None if f["e"] is None else f["e"].t
+        k._fused_adam_step(a["m"].t, a["ms"].t, a["v"].t, a["vs"].t, a["p"].t, a["g"].t, ecc(a), 1e-3, 0.9, 0.999, 1e-8, 1e-5, True, 1)
+        before = [{name: fenced.raw.clone() for name, fenced in f.items() if fenced is not None} for f in (a, b)]
+        tensors = [StepTensors(f["p"].t, f["g"].t, ecc(f), f["m"].t, f["ms"].t, f["v"].t, f["vs"].t) for f in (a, b)]
+        ecc_bytes = 0 if ecc_dtype is None else torch.empty(0, dtype=ecc_dtype).element_size()
+        plan = BucketPlan("adam", dtype, ecc_bytes, True, tensors)
+        plan.launch_streams_copy()
+        plan.launch_streams_copy()
+        torch.cuda.synchronize()
+        for f, old in zip((a, b), before):
+            for name, raw in old.items():
+                assert torch.equal(f[name].raw, raw), f"n={n} {dtype}: `{name}` changed under the access-mix copy"
+
+
 def test_randomised_configurations_match_oracle():
     """400 seeded random configurations (kernel family, dtype, ECC width, quantisation, length, misalignment,
     hyper-parameters over several decades, gradient and weight scales from 1e-7 to 1e2, sparse gradients), three
