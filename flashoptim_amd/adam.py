@@ -25,7 +25,7 @@ class FlashAdam(FlashOptimizer):
         exact_update: keyword-only, not in the reference (default: the ``FLASHOPTIM_EXACT_ADAM`` environment variable,
             else False).  Evaluate the update operation by operation as the reference writes it for bf16 / fp16
             parameters too (fp32 parameters always are): master weights and state codes then equal an IEEE
-            evaluation of the reference's formulas bit for bit, at 9-14 % less throughput.  With False the bias
+            evaluation of the reference's formulas bit for bit, at 5-11 % less throughput.  With False the bias
             corrections and the learning rate are folded into two constants, which leaves 1e-4 (24-bit masters) to
             2e-2 (32-bit masters) of the master weights more than one unit of master precision away.
     """

@@ -126,11 +126,18 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT = AdamExact<D
     using Hyper = AdamHyper;
     static constexpr int kLutTables = ECCB == 1 ? 2 : (QUANT ? 1 : 0);  // LDS code tables (fo_device.h)
     static constexpr int kDtype = DT;
-    // measured on MI355X with the 8B-parameter step and this file's ILP-oriented instruction schedule: 16-17
-    // resident workgroups per compute unit for 2-byte parameters (3.6-4.6 KiB of loads per wavefront; 15 and 18
-    // are two to three points worse on the 8B list, a flat tensor does not care between 15 and 17), 18-20 for fp32
-    // parameters (2.5 KiB) and for the arithmetic-bound operation-by-operation update on 2-byte parameters.
-    static constexpr int kWorkgroupsPerCu = (DT == DT_F32 || EXACT) ? 20 : 16;
+    // measured on MI355X with the 8B-parameter step and this file's ILP-oriented instruction schedule, over the
+    // residencies the LDS units allow (fo_step.h): 16 for 2-byte parameters (3.6-4.6 KiB of loads per wavefront; 14
+    // and 18 are two to three points worse on the 8B list), 18 for fp32 parameters (2.5 KiB per wavefront), 20 for
+    // the arithmetic-bound operation-by-operation update on 2-byte parameters.
+    // Wavefronts per SIMD: left alone, a compute unit spreads its sixteen wavefronts unevenly over the SIMDs on most
+    // boxes of the pool.  A cap of four (an even spread) gains 0.6 points there with 0- and 1-byte ECC and costs
+    // nothing on the other boxes.  With 2-byte ECC it gains two points on the former and loses 1.5 on the latter, and
+    // a cap of five is as erratic, so that variant stays uncapped, like fp32 (a cap costs a point there).  The
+    // operation-by-operation update on 2-byte parameters gains two points from its cap of five on every box.
+    static constexpr bool kNarrowExact = EXACT && DT != DT_F32;
+    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 18 : (kNarrowExact ? 20 : 16);
+    static constexpr int kMaxWavesPerSimd = DT == DT_F32 ? 8 : (kNarrowExact ? 5 : (ECCB == 2 ? 8 : 4));
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {
@@ -154,9 +161,10 @@ template <int DT, int ECCB, bool QUANT> struct AdamStreamsOp {
     using Hyper = StreamsHyper;
     static constexpr int kLutTables = 0;
     static constexpr int kDtype = DT;
-    // where this copy streams fastest on MI355X with the 8B-parameter list: 16-17 with 1-byte ECC (14-15 and 18-20
-    // are three to four points slower), 14-15 with 2-byte ECC (16-17 one point slower)
-    static constexpr int kWorkgroupsPerCu = ECCB == 2 ? 15 : 16;
+    // where this copy streams fastest on MI355X with the 8B-parameter list: 16 with 1-byte ECC (14 and 18 are three
+    // to four points slower), 14 with 2-byte ECC (16 one point slower)
+    static constexpr int kWorkgroupsPerCu = ECCB == 2 ? 14 : 16;
+    static constexpr int kMaxWavesPerSimd = 8;
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {

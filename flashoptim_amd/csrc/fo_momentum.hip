@@ -87,10 +87,13 @@ template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumOp {
     using Hyper = MomentumHyper;
     static constexpr int kLutTables = ECCB == 1 ? 2 : ((QUANT && KIND != KIND_PLAIN) ? 1 : 0);  // LDS code tables (fo_device.h)
     static constexpr int kDtype = DT;
-    // measured on MI355X (3 KiB of loads per wavefront): 24 best for the 8B list, 26-30 for 4096 ragged tensors.
-    // (The ILP-oriented schedule that fo_adam.hip is built with gains 1-2 points on the 8B list at 18-20 resident
+    // measured on MI355X (3 KiB of loads per wavefront) over the residencies the LDS units allow (fo_step.h: 18, 21,
+    // 25, 32 around here): the 8B list is as fast at 21 as at 25, 4096 ragged tensors need 25 or more; capping the
+    // wavefronts per SIMD at 6 or 7 changes nothing measurable.
+    // (The ILP-oriented schedule that fo_adam.hip is built with gains 1-2 points on the 8B list at 18-21 resident
     // workgroups and loses as much on the ragged list, which wants more than the 24 that its 80 VGPRs allow.)
-    static constexpr int kWorkgroupsPerCu = 26;
+    static constexpr int kWorkgroupsPerCu = 25;
+    static constexpr int kMaxWavesPerSimd = 8;
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = MomentumRaw<DT, ECCB, QUANT, KIND>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {

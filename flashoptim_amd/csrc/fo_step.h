@@ -278,8 +278,12 @@ __device__ __forceinline__ void run_span(const TensorPtrs& t, int64_t base, bool
     }
 }
 
+// Op::kMaxWavesPerSimd caps the wavefronts a SIMD holds (8 = the hardware's own limit, i.e. no cap): the code object
+// then declares enough registers that no SIMD takes more, and the compute unit's resident workgroups (capped through
+// LDS, fo_host::plan_residency) spread evenly over its four SIMDs instead of piling up on some of them.
+#define FO_WAVES_ATTR __attribute__((amdgpu_waves_per_eu(1, Op::kMaxWavesPerSimd)))
 template <class Op>
-__global__ __launch_bounds__(kBlockThreads) void step_single_kernel(TensorPtrs t, typename Op::Hyper h) {
+__global__ __launch_bounds__(kBlockThreads) FO_WAVES_ATTR void step_single_kernel(TensorPtrs t, typename Op::Hyper h) {
     __shared__ __align__(16) float lut[StepLut<Op::kLutTables>::kFloats];
     const int64_t base = (int64_t)blockIdx.x * Span<Op>::kElems;
     if constexpr (Op::kLutTables > 0) StepLut<Op::kLutTables>::fill(lut, kStepTables<Op::kDtype>.v);
@@ -288,7 +292,7 @@ __global__ __launch_bounds__(kBlockThreads) void step_single_kernel(TensorPtrs t
 
 // Workgroup b works on chunk b / kPerTile and takes span b % kPerTile of each of the chunk's tiles.
 template <class Op>
-__global__ __launch_bounds__(kBlockThreads) void step_multi_kernel(const fo_tensor_desc* __restrict__ descs,
+__global__ __launch_bounds__(kBlockThreads) FO_WAVES_ATTR void step_multi_kernel(const fo_tensor_desc* __restrict__ descs,
                                                                    const fo_chunk* __restrict__ chunks, typename Op::Hyper h) {
     __shared__ __align__(16) float lut[StepLut<Op::kLutTables>::kFloats];
     constexpr int kPerTile = Span<Op>::kPerTile;
@@ -349,14 +353,18 @@ inline int validate_multi(const fo_tensor_desc* descs, int64_t n_tensors, const 
 
 // Streaming from HBM degrades when a compute unit keeps too many bytes in flight, and a step wavefront has
 // several KiB of loads outstanding.  Each kernel family therefore names the number of workgroups it wants
-// resident per compute unit (Op::kWorkgroupsPerCu, the middle of the plateau measured on MI355X) and the launch
-// requests enough unused dynamic LDS to cap the residency there.  The request is derived from the device's LDS
-// per compute unit and confirmed with the runtime's occupancy query, once per kernel and device.
+// resident per compute unit (Op::kWorkgroupsPerCu, the best of those measured on MI355X) and the launch requests
+// enough unused dynamic LDS to cap the residency there.  gfx950 hands out LDS in units of 320 dwords, 128 of them
+// per compute unit, so the counts that can be reached this way are 128 / k: ... 12, 14, 16, 18, 21, 25, 32 (measured
+// durations fall on exactly these plateaus, whatever finer count the runtime's occupancy query grants).  A family
+// may also cap the wavefronts per SIMD (Op::kMaxWavesPerSimd); the query reports the smaller of the two limits.
 struct Residency {
     int target = 0;    // workgroups per compute unit asked for
-    int achieved = 0;  // what the occupancy query reports with `dynamic_lds`
+    int achieved = 0;  // what the LDS units and the occupancy query allow with `dynamic_lds`
     unsigned dynamic_lds = 0;
 };
+
+constexpr long kLdsUnitBytes = 1280;
 
 template <class Kernel>
 Residency plan_residency(Kernel kernel, int target, int static_lds) {
@@ -366,23 +374,19 @@ Residency plan_residency(Kernel kernel, int target, int static_lds) {
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&lds_per_cu, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, dev) != hipSuccess || lds_per_cu <= 0)
         return r;
-    auto query = [&](long bytes) {
-        int n = 0;
-        const long dyn = bytes > static_lds ? bytes - static_lds : 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, fo::kBlockThreads, (size_t)dyn) != hipSuccess) n = 0;
-        return n;
-    };
-    // half-way between the footprints that would admit target and target + 1 workgroups, so that neither the
-    // allocation granularity nor a few bytes of static LDS tip the count
-    long bytes = ((long)lds_per_cu / target + (long)lds_per_cu / (target + 1)) / 2 / 256 * 256;
-    int got = query(bytes);
-    for (int tries = 0; tries < 64 && got != target && got > 0; ++tries) {
-        bytes += got > target ? 256 : -256;
-        if (bytes <= static_lds) { bytes = static_lds; got = query(bytes); break; }
-        got = query(bytes);
-    }
-    r.achieved = got;
-    r.dynamic_lds = (unsigned)(bytes > static_lds ? bytes - static_lds : 0);
+    // the most LDS units per workgroup that still admit `target` workgroups
+    const long units_per_cu = lds_per_cu / kLdsUnitBytes;
+    long units = units_per_cu / target;
+    const long least = (static_lds + kLdsUnitBytes - 1) / kLdsUnitBytes;
+    if (units < least) units = least;
+    if (units < 1) units = 1;
+    const long bytes = units * kLdsUnitBytes;
+    const long dyn = bytes > static_lds ? bytes - static_lds : 0;
+    int granted = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&granted, kernel, fo::kBlockThreads, (size_t)dyn) != hipSuccess) granted = 0;
+    const long by_units = units_per_cu / units;
+    r.achieved = granted < by_units ? granted : (int)by_units;
+    r.dynamic_lds = (unsigned)dyn;
     return r;
 }
 

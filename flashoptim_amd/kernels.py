@@ -268,7 +268,7 @@ def _fused_adam_step(
 
     ``exact_update`` (not in the reference): evaluate the update operation by operation as the reference writes it,
     for bf16 / fp16 parameters too (fp32 parameters always are); every output bit then equals an IEEE evaluation of
-    the reference's formulas, at 9-14 % less throughput."""
+    the reference's formulas, at 5-11 % less throughput."""
     _check_group_size(group_size)
     n = param.numel()
     if n == 0:

@@ -145,7 +145,7 @@ int fo_multi_adam_step_static(const fo_tensor_desc *host_descs, int64_t n_tensor
  * points do this for fp32 parameters only; for bf16 / fp16 parameters they fold the bias corrections and the
  * learning rate into two constants (one reciprocal per element), which leaves 1e-4 (24-bit masters) to 2e-2
  * (32-bit masters) of the master weights more than one unit of master precision away from that evaluation, and is
- * roughly 10-15 % faster.  Same arguments and errors as the plain entry points.  The reference has one kernel and no such
+ * roughly 5-12 % faster.  Same arguments and errors as the plain entry points.  The reference has one kernel and no such
  * choice; these are for callers who want the stricter arithmetic.
  */
 int fo_adam_step_exact(void *mom, void *mom_scales, void *var, void *var_scales, void *param, const void *grad,
