@@ -15,8 +15,8 @@ Workloads (``--workload``):
   llama8b-mwb24-exact / llama8b-mwb32-exact
                   the same with FlashAdamW(exact_update=True): the update evaluated operation by operation
                   (bit-exact with the CPU oracle), to show what that costs.
-  llama8b-mwb24-streams / llama8b-mwb32-streams
-                  the memory accesses of those two steps without the arithmetic (every stream read and written back
+  llama8b-mwb24-streams / llama8b-mwb32-streams / llama8b-fp32-streams
+                  the memory accesses of the bf16 steps and of the fp32 step without the arithmetic (every stream read and written back
                   unchanged by the step kernels' own access code): the rate this access mix can reach on the box,
                   to be read next to the step's (``value`` counts the same parameters and bytes as the step).
   flat-2p30       one flat bf16 tensor of 2^30 elements, FlashAdamW, master_weight_bits=24.
@@ -147,21 +147,24 @@ def build_workload(name: str, device):
                          + ("exact_update=True (operation-by-operation update), " if exact else "")
                          + "gradients redrawn per step (3 rotating sets)",
                     launch="one multi-tensor launch per step", optimizer="FlashAdamW", mwb=mwb)
-    if name in ("llama8b-mwb24-streams", "llama8b-mwb32-streams"):
+    if name in ("llama8b-mwb24-streams", "llama8b-mwb32-streams", "llama8b-fp32-streams"):
         from flashoptim_amd.launcher import BucketPlan
 
         shapes = llama3_8b_shapes()
         g = torch.Generator().manual_seed(2)
         scales = (10.0 ** (torch.rand(len(shapes), generator=g) * 2 - 1)).tolist()
-        params = make_params(shapes, torch.bfloat16, device, scales)
-        mwb = 24 if "mwb24" in name else 32
+        fp32 = "fp32" in name
+        mwb = None if fp32 else (24 if "mwb24" in name else 32)
+        ecc_bytes = {None: 0, 24: 1, 32: 2}[mwb]
+        dtype = torch.float32 if fp32 else torch.bfloat16
+        params = make_params(shapes, dtype, device, scales)
         opt = fo.FlashAdamW(params, master_weight_bits=mwb, **hp)
         rotating_gradients(params, opt.step, device, scales, sets=1)()  # one real step: states exist and hold values
         planned = [opt._plan_param(p, opt.param_groups[0]) for p in params]
-        plan = BucketPlan("adam", torch.bfloat16, 1 if mwb == 24 else 2, True, [t for _, t in planned])
-        return dict(params=params, opt=None, step=plan.launch_streams_copy, bpp=bytes_per_param(2, 1 if mwb == 24 else 2, 2),
-                    desc=f"memory accesses of the FlashAdamW step (master_weight_bits={mwb}) on the Llama-3-8B-shaped "
-                         "list without its arithmetic: every stream read and written back unchanged",
+        plan = BucketPlan("adam", dtype, ecc_bytes, True, [t for _, t in planned])
+        return dict(params=params, opt=None, step=plan.launch_streams_copy, bpp=bytes_per_param(4 if fp32 else 2, ecc_bytes, 2),
+                    desc=f"memory accesses of the FlashAdamW step ({'fp32 parameters' if fp32 else f'master_weight_bits={mwb}'}) on the "
+                         "Llama-3-8B-shaped list without its arithmetic: every stream read and written back unchanged",
                     launch="one multi-tensor launch per step", optimizer=None, mwb=mwb, keep=(opt, plan))
     if name in ("llama8b-lion", "llama8b-sgdw"):
         shapes = llama3_8b_shapes()

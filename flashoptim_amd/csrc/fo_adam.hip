@@ -162,8 +162,9 @@ template <int DT, int ECCB, bool QUANT> struct AdamStreamsOp {
     static constexpr int kLutTables = 0;
     static constexpr int kDtype = DT;
     // where this copy streams fastest on MI355X with the 8B-parameter list: 16 with 1-byte ECC (14 and 18 are three
-    // to four points slower), 14 with 2-byte ECC (16 one point slower)
-    static constexpr int kWorkgroupsPerCu = ECCB == 2 ? 14 : 16;
+    // to four points slower), 14 with 2-byte ECC (16 one point slower); fp32 parameters (256 elements and 2.5 KiB per
+    // wavefront, the codes as 4-byte loads) want every slot: 32 (79.6 %; 25: 79.2 %, 18: 74.6 %)
+    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 32 : (ECCB == 2 ? 14 : 16);
     static constexpr int kMaxWavesPerSimd = 8;
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
