@@ -22,6 +22,8 @@ Workloads (``--workload``):
   flat-2p30       one flat bf16 tensor of 2^30 elements, FlashAdamW, master_weight_bits=24.
   llama8b-lion / llama8b-sgdw
                   the same parameter list under FlashLion / FlashSGDW (one quantised moment), master_weight_bits=24.
+  llama8b-lion-streams / ragged-streams
+                  the momentum kernels' loads and stores without their arithmetic, on those two lists.
   ragged-lion / ragged-sgdw
                   4096 bf16 tensors with log-uniform lengths in [1, 2^24] (~1e9 parameters), FlashLion / FlashSGDW.
   llama8b-fp32-release
@@ -129,6 +131,20 @@ def rotating_gradients(params, step, device, grad_scales=None, sets=3):
     return run
 
 
+def momentum_streams_workload(params, opt, what):
+    """The momentum kernels' loads and stores without their arithmetic, on the launch tables of `opt` after one real
+    step (so that the states exist and hold values)."""
+    from flashoptim_amd.launcher import BucketPlan
+
+    opt.step()
+    planned = [opt._plan_param(p, opt.param_groups[0]) for p in params]
+    plan = BucketPlan("momentum", torch.bfloat16, 1, True, [t for _, t in planned])
+    return dict(params=params, opt=None, step=plan.launch_streams_copy, bpp=bytes_per_param(2, 1, 1),
+                desc=f"memory accesses of the FlashLion / FlashSGDW step (master_weight_bits=24) on {what} without the "
+                     "arithmetic: every stream read and written back unchanged",
+                launch="one multi-tensor launch per step", optimizer=None, mwb=24, keep=(opt, plan))
+
+
 def build_workload(name: str, device):
     import flashoptim_amd as fo
 
@@ -166,15 +182,17 @@ def build_workload(name: str, device):
                     desc=f"memory accesses of the FlashAdamW step ({'fp32 parameters' if fp32 else f'master_weight_bits={mwb}'}) on the "
                          "Llama-3-8B-shaped list without its arithmetic: every stream read and written back unchanged",
                     launch="one multi-tensor launch per step", optimizer=None, mwb=mwb, keep=(opt, plan))
-    if name in ("llama8b-lion", "llama8b-sgdw"):
+    if name in ("llama8b-lion", "llama8b-sgdw", "llama8b-lion-streams"):
         shapes = llama3_8b_shapes()
         g = torch.Generator().manual_seed(2)
         scales = (10.0 ** (torch.rand(len(shapes), generator=g) * 2 - 1)).tolist()
         params = make_params(shapes, torch.bfloat16, device, scales)
-        if name == "llama8b-lion":
+        if name in ("llama8b-lion", "llama8b-lion-streams"):
             opt = fo.FlashLion(params, lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1, master_weight_bits=24)
         else:
             opt = fo.FlashSGDW(params, momentum=0.9, lr=1e-2, weight_decay=1e-4, master_weight_bits=24)
+        if name == "llama8b-lion-streams":
+            return momentum_streams_workload(params, opt, "Llama-3-8B-shaped parameter list, bf16")
         return dict(params=params, opt=opt, step=opt.step, bpp=bytes_per_param(2, 1, 1),
                     desc=f"Llama-3-8B-shaped parameter list, bf16, {type(opt).__name__}, master_weight_bits=24",
                     launch="one multi-tensor launch per step", optimizer=type(opt).__name__, mwb=24)
@@ -185,7 +203,7 @@ def build_workload(name: str, device):
                     desc="one flat bf16 tensor of 2^30 elements, FlashAdamW, master_weight_bits=24, gradients redrawn per "
                          "step (3 rotating sets)",
                     launch="one single-tensor launch per step", optimizer="FlashAdamW", mwb=24)
-    if name in ("ragged-lion", "ragged-sgdw"):
+    if name in ("ragged-lion", "ragged-sgdw", "ragged-streams"):
         lens = ragged_lengths()
         torch.manual_seed(3)
         # parameters and gradients are carved from two flat buffers at 512-byte aligned offsets (what torch's
@@ -210,10 +228,12 @@ def build_workload(name: str, device):
             p = torch.nn.Parameter(flat_p[o:o + n])
             p.grad = flat_g[o:o + n]
             params.append(p)
-        if name == "ragged-lion":
+        if name in ("ragged-lion", "ragged-streams"):
             opt = fo.FlashLion(params, lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1, master_weight_bits=24)
         else:
             opt = fo.FlashSGDW(params, momentum=0.9, lr=1e-2, weight_decay=1e-4, master_weight_bits=24)
+        if name == "ragged-streams":
+            return momentum_streams_workload(params, opt, "4096 bf16 tensors, lengths log-uniform in [1, 2^24]")
         return dict(params=params, opt=opt, step=opt.step, bpp=bytes_per_param(2, 1, 1),
                     desc="4096 bf16 tensors, lengths log-uniform in [1, 2^24], Student-t(3) gradients, "
                          + type(opt).__name__ + ", master_weight_bits=24",

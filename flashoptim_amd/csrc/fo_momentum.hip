@@ -105,6 +105,39 @@ template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumOp {
     }
 };
 
+
+// The momentum step's memory accesses without its arithmetic (see AdamStreamsOp in fo_adam.hip): parameters,
+// gradients, ECC, the moment's codes and scales are loaded and everything but the gradients is stored back unchanged
+// by the step's own load / store code.
+struct MomentumStreamsHyper { uint32_t mask; };
+
+template <int DT, int ECCB, bool QUANT> struct MomentumStreamsOp {
+    using Hyper = MomentumStreamsHyper;
+    static constexpr int kLutTables = 0;
+    static constexpr int kDtype = DT;
+    // measured on MI355X: the 8B-parameter list streams fastest at 14 (83.2 %; 16: 82.0 %, 18: 79.6 %), 4096 ragged
+    // tensors at 16 (81.8 %; 14: 80.2 %, 18: 81.5 %)
+    static constexpr int kWorkgroupsPerCu = 16;
+    static constexpr int kMaxWavesPerSimd = 8;
+    static constexpr int kEpl = DTypeInfo<DT>::epl;
+    using Raw = MomentumRaw<DT, ECCB, QUANT, KIND_SGD>;
+    template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {
+        momentum_load<DT, ECCB, QUANT, KIND_SGD, FAST>(t, w, r);
+    }
+    template <int FAST>
+    __device__ __forceinline__ static void finish(const TensorPtrs& t, Where w, Raw& r, const Hyper& h, const float*) {
+        constexpr int PB = DTypeInfo<DT>::bytes;
+#pragma unroll
+        for (int i = 0; i < Pack<PB, kEpl>::kDwords; ++i) r.p.w[i] ^= r.g.w[i] & h.mask;
+        store_lane<PB, kEpl, FAST>(r.p, t.param, w, t.n);
+        store_lane<ECCB, kEpl, FAST>(r.e, t.ecc, w, t.n);
+        store_lane<Raw::SB, kEpl, FAST>(r.m, t.mom, w, t.n);
+        if constexpr (QUANT) {
+            if ((FAST == kVector || w.first() < t.n) && (threadIdx.x & (32 / kEpl - 1)) == 0) store_scale(t.mom_scales, w, r.sm);
+        }
+    }
+};
+
 }  // namespace fo
 
 namespace {
@@ -154,6 +187,14 @@ int fo_multi_sgd_plain_step(const fo_tensor_desc* descs, int64_t n_tensors, cons
     if (n_chunks == 0) return 0;
     MultiLauncher<fo::MomentumHyper> L{descs, chunks, n_chunks, make_momentum_hyper(lr, 0.0f, 1.0f, weight_decay, decoupled, 0), (hipStream_t)stream};
     return dispatch<PlainOp>(dtype, ecc_bytes, 0, L);
+}
+
+int fo_multi_momentum_streams_copy(const fo_tensor_desc* descs, int64_t n_tensors, const fo_chunk* chunks, int64_t n_chunks,
+                                   int dtype, int ecc_bytes, int quantized, void* stream) {
+    if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
+    if (n_chunks == 0) return 0;
+    MultiLauncher<fo::MomentumStreamsHyper> L{descs, chunks, n_chunks, fo::MomentumStreamsHyper{0u}, (hipStream_t)stream};
+    return dispatch<fo::MomentumStreamsOp>(dtype, ecc_bytes, quantized, L);
 }
 
 int fo_momentum_step_residency(int dtype, int ecc_bytes, int quantized, int kind, int multi, int* target, int* achieved,

@@ -190,16 +190,17 @@ class BucketPlan:
         _native.check(rc, "fo_multi_sgd_plain_step" if self.kind == "plain" else f"fo_multi_{self.kind}_step")
 
     def launch_streams_copy(self) -> None:
-        """Measurement aid (Adam buckets): read every stream of the bucket and write it back unchanged with the step
-        kernels' access code, without the step's arithmetic; shows what rate the step's access mix can reach."""
-        if self.kind != "adam":
-            raise ValueError("the access-mix copy exists for Adam buckets only")
+        """Measurement aid (Adam and momentum buckets): read every stream of the bucket and write it back unchanged
+        with the step kernels' access code, without the step's arithmetic; shows what rate the step's access mix can
+        reach."""
+        if self.kind not in ("adam", "momentum"):
+            raise ValueError("the access-mix copy exists for Adam and momentum buckets only")
         if self.n_chunks == 0:
             return
         with _native.device_guard(self.device):
             if self._dirty:
                 self._upload()
-            rc = _native.lib().fo_multi_adam_streams_copy(
-                self.descs_dev.data_ptr(), self.n_tensors, self.chunks_dev.data_ptr(), self.n_chunks,
-                DTYPE_CODE[self.dtype], self.ecc_bytes, int(self.quantized), _native.current_stream_ptr(self.device))
-        _native.check(rc, "fo_multi_adam_streams_copy")
+            entry = getattr(_native.lib(), f"fo_multi_{self.kind}_streams_copy")
+            rc = entry(self.descs_dev.data_ptr(), self.n_tensors, self.chunks_dev.data_ptr(), self.n_chunks,
+                       DTYPE_CODE[self.dtype], self.ecc_bytes, int(self.quantized), _native.current_stream_ptr(self.device))
+        _native.check(rc, f"fo_multi_{self.kind}_streams_copy")

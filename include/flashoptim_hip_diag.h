@@ -31,6 +31,9 @@ int fo_copy_bytes(void *dst, const void *src, int64_t n_bytes, void *stream);
  */
 int fo_multi_adam_streams_copy(const fo_tensor_desc *descs, int64_t n_tensors, const fo_chunk *chunks, int64_t n_chunks,
                                int dtype, int ecc_bytes, int quantized, void *stream);
+/* The same for the momentum kernels' streams (parameters, gradients, ECC, one moment's codes and scales). */
+int fo_multi_momentum_streams_copy(const fo_tensor_desc *descs, int64_t n_tensors, const fo_chunk *chunks,
+                                   int64_t n_chunks, int dtype, int ecc_bytes, int quantized, void *stream);
 
 /*
  * Residency plan of a step kernel on the current device: the workgroups per compute unit the kernel family asks

@@ -497,9 +497,10 @@ def test_kernels_never_write_outside_their_tensors(n):
 
 @pytest.mark.parametrize("n", [1, 33, 511, 4096, 4097, 3 * 4096 + 40, 1 << 20])
 def test_access_mix_copy_changes_no_byte(n):
-    """The measurement kernel that runs the Adam step's loads and stores without its arithmetic leaves parameters,
-    gradients, ECC, codes and scales exactly as they were, and the bytes next to them untouched (bf16 with both ECC
-    widths, fp16, fp32; two tensors per launch, one of them after a real step so that no stream is all zero)."""
+    """The measurement kernels that run the Adam and the momentum step's loads and stores without the arithmetic
+    leave parameters, gradients, ECC, codes and scales exactly as they were, and the bytes next to them untouched
+    (bf16 with both ECC widths, fp16, fp32; two tensors per launch, one of them after a real step so that no stream
+    is all zero)."""
     k = _k()
     from flashoptim_amd.launcher import BucketPlan, StepTensors
 
@@ -523,6 +524,7 @@ def test_access_mix_copy_changes_no_byte(n):
         plan = BucketPlan("adam", dtype, ecc_bytes, True, tensors)
         plan.launch_streams_copy()
         plan.launch_streams_copy()
+        BucketPlan("momentum", dtype, ecc_bytes, True, tensors).launch_streams_copy()
         torch.cuda.synchronize()
         for f, old in zip((a, b), before):
             for name, raw in old.items():
