@@ -330,37 +330,104 @@ def measured_traffic(workload: str):
 
 def parity_subcheck(device, ecc_dtype=torch.int8, steps: int = 4, exact_update: bool = False):
     """HIP step against the CPU oracle on 2^20 and 2^20 + 17 bf16 elements (parameters N(0, 0.02), gradients
-    N(0, 1e-3) redrawn per step, FlashAdamW hyper-parameters of the throughput run), outside the timed region.
-    Reports the raw share of moment codes that differ (never by more than one step) per step, the first included,
-    and the share of master weights more than one unit of master precision away with no allowance."""
+    N(0, 1e-3) redrawn per step, FlashAdamW hyper-parameters of the throughput run), outside the timed region, every
+    step from identical inputs.  Nothing is allowed for: the figures are raw counts.  Per step: the share of moment
+    codes and of fp16 group scales that differ at all, the share of master weights (narrow parameter + correction
+    code) more than one unit of master precision from the oracle's, the largest such difference in units, and the
+    share that is exactly one unit apart (within the bar)."""
     from flashoptim_amd import kernels as k
     from oracle import torch_oracle as T
     from tests import parity
 
-    out = {"sizes": [], "code_mismatch_fraction_per_step": [], "master_beyond_one_unit_per_step": []}
+    out = {"sizes": [], "code_mismatch_fraction_per_step": [], "scale_mismatch_fraction_per_step": [],
+           "master_beyond_one_unit_per_step": [], "master_max_units_per_step": [], "master_one_unit_apart_per_step": [],
+           "narrow_beyond_one_ulp_per_step": []}
     for n in (1 << 20, (1 << 20) + 17):
         p = (torch.randn(n, generator=torch.Generator().manual_seed(0)) * 0.02).to(torch.bfloat16)
         ecc = torch.zeros(n, dtype=ecc_dtype)
         m, v = T.MomentState.zeros(n, True, True, torch.bfloat16), T.MomentState.zeros(n, False, True, torch.bfloat16)
         gp, gecc = p.to(device), ecc.to(device)
         gm, gms, gv, gvs = m.codes.to(device), m.scales.to(device), v.codes.to(device), v.scales.to(device)
-        rates, beyond = [], []
+        rows = {key: [] for key in out if key != "sizes"}
         for step in range(1, steps + 1):
             g = (torch.randn(n, generator=torch.Generator().manual_seed(1000 + step)) * 1e-3).to(torch.bfloat16)
             k._fused_adam_step(gm, gms, gv, gvs, gp, g.to(device), gecc, 1e-3, 0.9, 0.999, 1e-8, 0.01 * 1e-3, True, step,
                                exact_update=exact_update)
-            info = T.adam_step_ref(m, v, p, g, ecc, 1e-3, 0.9, 0.999, 1e-8, 0.01 * 1e-3, True, step)
-            rates.append(max(parity.check_codes(gm, m.codes, "bench m"), parity.check_codes(gv, v.codes, "bench v")))
-            parity.check_scales(gms, m.scales, "bench m scales")
-            parity.check_scales(gvs, v.scales, "bench v scales")
-            beyond.append(parity.check_master(gp, gecc, p, ecc, "bench master", step_size=info["update_scale"])[1])
+            T.adam_step_ref(m, v, p, g, ecc, 1e-3, 0.9, 0.999, 1e-8, 0.01 * 1e-3, True, step)
+            codes = sum(int((a.cpu().view(torch.uint8) != b.view(torch.uint8)).sum()) for a, b in ((gm, m.codes), (gv, v.codes)))
+            scales = sum(int((a.cpu().view(torch.int16) != b.view(torch.int16)).sum()) for a, b in ((gms, m.scales), (gvs, v.scales)))
+            narrow, master = parity.master_difference(gp, gecc, p, ecc)
+            rows["code_mismatch_fraction_per_step"].append(codes / (2 * n))
+            rows["scale_mismatch_fraction_per_step"].append(scales / (2 * m.scales.numel()))
+            rows["master_beyond_one_unit_per_step"].append(float((master > 1.0 + 1e-9).double().mean()))
+            rows["master_max_units_per_step"].append(float(master.max()))
+            rows["master_one_unit_apart_per_step"].append(float(((master > 0) & (master <= 1.0 + 1e-9)).double().mean()))
+            rows["narrow_beyond_one_ulp_per_step"].append(float((narrow > 1.0 + 1e-9).double().mean()))
             for dst, src in ((p, gp), (ecc, gecc), (m.codes, gm), (m.scales, gms), (v.codes, gv), (v.scales, gvs)):
                 dst.copy_(src.cpu())  # the next comparison starts from identical inputs
         out["sizes"].append(n)
-        out["code_mismatch_fraction_per_step"].append(rates)
-        out["master_beyond_one_unit_per_step"].append(beyond)
-    out["first_step_codes_identical"] = all(r[0] == 0.0 for r in out["code_mismatch_fraction_per_step"])
+        for key, row in rows.items():
+            out[key].append(row)
+    flat = lambda key: [x for row in out[key] for x in row]
+    out["codes_and_scales_bit_exact"] = not any(flat("code_mismatch_fraction_per_step") + flat("scale_mismatch_fraction_per_step"))
+    out["within_tolerance"] = out["codes_and_scales_bit_exact"] and not any(flat("master_beyond_one_unit_per_step") + flat("narrow_beyond_one_ulp_per_step"))
     return out
+
+
+def measure(work, steps: int, warmup: int) -> dict:
+    """W warm-up steps, then exactly K steps between two synchronisations.  Returns the timings of one workload."""
+    step = work["step"]
+    total = sum(p.numel() for p in work["params"])
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    # Events on the launch stream (torch's current stream) around the K timed steps, without per-step event overhead
+    # (several percent of a 1.6 ms step).  The device idles while the host prepares the first timed step (1 ms for a
+    # list of 4096 tensors), so the kernels' average duration is taken from the end of the first step to the end of
+    # the last, where the host runs ahead of the device; the wall clock behind `value` includes that lead-in.
+    first, second, last = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+    t0 = time.perf_counter()
+    first.record()
+    for i in range(steps):
+        step()
+        if i == 0:
+            second.record()
+    last.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / steps
+    avg_device_ms = second.elapsed_time(last) / (steps - 1) if steps > 1 else first.elapsed_time(last)
+    step_bytes = work.get("copy_bytes", total * work["bpp"])
+    achieved = step_bytes / (avg_device_ms * 1e-3) / 1e9
+    return dict(total=total, ms_per_step=ms_per_step, avg_device_ms=avg_device_ms, step_bytes=step_bytes, achieved=achieved,
+                frac=achieved / HBM_PEAK_GBPS, frac_wall=step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                with_lead_in_ms=first.elapsed_time(last) / steps)
+
+
+# The other configurations of the baseline, run after the default workload (a few steps each): the flat 2^30 tensor,
+# the 8B list with 32-bit masters, the 4096 ragged tensors under Lion and SGDW, the fp32 gradient-release order.
+SECONDARY = ("flat-2p30", "llama8b-mwb32", "ragged-lion", "ragged-sgdw", "llama8b-fp32-release")
+
+
+def run_secondary(name: str, device, steps: int, warmup: int, parity: bool) -> dict:
+    work = build_workload(name, device)
+    t = measure(work, steps, warmup)
+    row = {"workload": name, "description": work["desc"], "n_params": t["total"], "steps": steps, "warmup": warmup,
+           "algorithmic_bytes_per_param": work["bpp"], "ms_per_step": t["ms_per_step"], "step_device_ms_avg": t["avg_device_ms"],
+           "params_per_s": t["total"] / (t["ms_per_step"] * 1e-3), "frac": t["frac"], "frac_wall": t["frac_wall"]}
+    if work.get("checkpoint_roundtrip"):
+        row["checkpoint_roundtrip_bit_exact"] = checkpoint_roundtrip(work, device)
+        row["checkpoint_bytes"] = work["checkpoint_bytes"]
+    adam_on_bf16 = work["optimizer"] == "FlashAdamW" and work["mwb"] in (24, 32)
+    mwb = work["mwb"]
+    work.clear()
+    del work
+    torch.cuda.empty_cache()
+    if adam_on_bf16 and parity:
+        sub = parity_subcheck(device, torch.int8 if mwb == 24 else torch.int16, steps=2)
+        row["parity"] = {key: sub[key] for key in ("codes_and_scales_bit_exact", "within_tolerance", "master_beyond_one_unit_per_step",
+                                                    "master_max_units_per_step")}
+    return row
 
 
 def main() -> None:
@@ -371,6 +438,8 @@ def main() -> None:
     ap.add_argument("--workload", default="llama8b-mwb24")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true", help="skip the HIP-vs-oracle sub-check that runs after the timed region")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="default workload only: skip the short runs of the other baseline configurations that follow it")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the optimizer step is shard-local and this build has no "
@@ -386,29 +455,8 @@ def main() -> None:
 
     work = build_workload(args.workload, device)
     step = work["step"]
-    total = sum(p.numel() for p in work["params"])
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    # Events on the launch stream (torch's current stream) around the K timed steps, without per-step event overhead
-    # (several percent of a 1.6 ms step).  The device idles while the host prepares the first timed step (1 ms for a
-    # list of 4096 tensors), so the kernels' average duration is taken from the end of the first step to the end of
-    # the last, where the host runs ahead of the device; the wall clock behind `value` includes that lead-in.
-    first, second, last = (torch.cuda.Event(enable_timing=True) for _ in range(3))
-    t0 = time.perf_counter()
-    first.record()
-    for i in range(args.steps):
-        step()
-        if i == 0:
-            second.record()
-    last.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    if args.steps > 1:
-        avg_device_ms = second.elapsed_time(last) / (args.steps - 1)
-    else:
-        avg_device_ms = first.elapsed_time(last)
+    t = measure(work, args.steps, args.warmup)
+    total, ms_per_step, avg_device_ms, step_bytes = t["total"], t["ms_per_step"], t["avg_device_ms"], t["step_bytes"]
 
     # a second pass with an event pair around every step, for the median and the fastest step (the pairs themselves
     # cost a few microseconds per step, which is why the averages above come from the pass without them)
@@ -420,8 +468,6 @@ def main() -> None:
     torch.cuda.synchronize()
     per_step = sorted(begin.elapsed_time(end) for begin, end in pairs)
 
-    step_bytes = work.get("copy_bytes", total * work["bpp"])
-    achieved = step_bytes / (avg_device_ms * 1e-3) / 1e9
     out = {
         "metric": "params updated/sec + achieved HBM GB/s (% peak), FlashAdamW step on 8B params",
         "value": total / (ms_per_step * 1e-3),
@@ -442,14 +488,14 @@ def main() -> None:
             "launch": work["launch"], "algorithmic_bytes_per_param": work["bpp"],
         },
         "roofline": {
-            "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS,
+            "bound": "hbm", "achieved": t["achieved"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": t["frac"],
             # the same algorithmic bytes over the host's wall clock per step (includes the host lead-in of the first step)
-            "frac_wall": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "frac_wall": t["frac_wall"],
             "traffic": measured_traffic(args.workload),
             "traffic_source": TRAFFIC_FILE + " (rocprofv3 FETCH_SIZE + WRITE_SIZE, recorded earlier; not measured by this run)"
                               if measured_traffic(args.workload) is not None else None,
-            "step_device_ms_avg": avg_device_ms, "step_device_ms_avg_with_lead_in": first.elapsed_time(last) / args.steps,
+            "step_device_ms_avg": avg_device_ms, "step_device_ms_avg_with_lead_in": t["with_lead_in_ms"],
             "step_device_ms_median": per_step[len(per_step) // 2], "step_device_ms_min": per_step[0],
             "algorithmic_bytes_per_step": step_bytes,
         },
@@ -459,10 +505,14 @@ def main() -> None:
         out["config"]["checkpoint_bytes"] = work["checkpoint_bytes"]
     adam_on_bf16 = work["optimizer"] == "FlashAdamW" and work["mwb"] in (24, 32)
     exact_update = args.workload.endswith("-exact")
-    del work
+    work.clear()
+    del work, step
+    torch.cuda.empty_cache()
     if adam_on_bf16 and not args.no_parity:
         out["parity"] = parity_subcheck(device, torch.int8 if out["config"]["master_weight_bits"] == 24 else torch.int16,
                                         exact_update=exact_update)
+    if args.workload == "llama8b-mwb24" and not args.no_secondary:
+        out["secondary"] = [run_secondary(name, device, steps=10, warmup=3, parity=not args.no_parity) for name in SECONDARY]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

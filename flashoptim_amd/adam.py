@@ -23,11 +23,13 @@ class FlashAdam(FlashOptimizer):
         weight_decay: L2 coefficient (default 0).
         quantize, compress_state_dict, master_weight_bits, check_numerics, fused: see :class:`FlashOptimizer`.
         exact_update: keyword-only, not in the reference (default: the ``FLASHOPTIM_EXACT_ADAM`` environment variable,
-            else False).  Evaluate the update operation by operation as the reference writes it for bf16 / fp16
-            parameters too (fp32 parameters always are): master weights and state codes then equal an IEEE
-            evaluation of the reference's formulas bit for bit, at 5-11 % less throughput.  With False the bias
-            corrections and the learning rate are folded into two constants, which leaves 1e-4 (24-bit masters) to
-            2e-2 (32-bit masters) of the master weights more than one unit of master precision away.
+            else False).  Evaluate the update operation by operation as the reference writes it on every element of
+            every variant: all outputs then equal an IEEE evaluation of the reference's formulas bit for bit.  With
+            False that already holds for fp32 parameters, 32-bit masters and fp16 parameters with 24-bit masters;
+            bf16 parameters with 24-bit masters and 2-byte parameters without master-weight correction fold the
+            bias corrections and the learning rate into two constants and redo operation by operation only the
+            elements whose update all but cancels the weight: moment codes and scales stay bit-identical, every
+            master weight stays within one unit of master precision (the correction code may differ by one step).
     """
 
     def __init__(

@@ -42,16 +42,14 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
     constexpr int EPL = DTypeInfo<DT>::epl;
     constexpr int PB = DTypeInfo<DT>::bytes;
     constexpr int SB = QUANT ? 1 : PB;
-    // the requantiser goes through the quick forms, every value verified (fo_math.h)
-    constexpr bool MAY_BE_QUICK = QUANT && (AdamQuickRequant<DT, ECCB>::value || EXACT);
-    constexpr bool EXACT_MOMENTS = EXACT || !AdamFoldedMoments<DT, ECCB>::value;
     const int64_t n = t.n;
     const bool live_group = FAST == kVector || w.first() < n;  // the lane owns at least one real element
     const float sm = f16_bits_to_f32(raw.sm), sv = f16_bits_to_f32(raw.sv);
-    const float sm_b1 = sm * h.b1, sv_b2 = sv * h.sqrt_b2_over_255;
 
     float p[EPL], m[EPL], r[EPL], v[EPL];
     read_master<DT, ECCB, EPL>(p, raw.p, raw.e, lut);
+    bool redo[EPL];
+    bool any_redo = false;
 
 #pragma unroll
     for (int k = 0; k < EPL; ++k) {
@@ -59,18 +57,37 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
         if constexpr (!DECOUPLED) g = g + p[k] * h.wd;                              // ref:2310-2311
         float mn, vn;
         if constexpr (QUANT) {
-            adam_moments_quantized<EXACT_MOMENTS>(g, lookup_mom(lut, byte_of<EPL>(raw.m, k)), sm, sm_b1,
-                                          (float)byte_of<EPL>(raw.v, k), sv, sv_b2, h, mn, vn);
+            adam_moments_quantized(g, lookup_mom(lut, byte_of<EPL>(raw.m, k)), sm, (float)byte_of<EPL>(raw.v, k), sv, h, mn, vn);
         } else {
             adam_moments_plain(g, widen<DT, EPL>(raw.m, k), widen<DT, EPL>(raw.v, k), h, mn, vn);
         }
-        float pk = p[k];
-        if constexpr (DECOUPLED) pk = pk * h.one_m_wd;                              // ref:2363-2364
-        // sqrt(v): the requantiser needs it (ref:2393) and the folded update shares it.  The folded update and the
-        // quick requantiser forms are content with the instruction's value.
-        const float rk = (QUANT || !EXACT) ? (MAY_BE_QUICK ? hw::sqrt(vn) : sqrt_corrected(vn)) : 0.0f;
-        p[k] = adam_apply<EXACT>(pk, mn, vn, rk, h);                                // ref:2368-2375
+        // sqrt(v) as the instruction gives it: the quick requantiser form and the folded update are content with it
+        const float rk = (QUANT || !EXACT) ? hw::sqrt(vn) : 0.0f;
+        if constexpr (EXACT) {
+            const float pk = DECOUPLED ? p[k] * h.one_m_wd : p[k];                  // ref:2363-2364
+            p[k] = adam_apply_exact(pk, mn, vn, h);                                 // ref:2368-2375
+        } else {
+            // folded update; `redo` marks the elements it cannot vouch for (fo_math.h).  The old weight stays in
+            // raw.p / raw.e for the repair below.
+            p[k] = adam_apply_folded<DECOUPLED>(p[k], mn, rk, h, AdamFoldedGuard<DT, ECCB>::value, redo[k]);
+            any_redo |= redo[k];
+        }
         m[k] = mn; r[k] = rk; v[k] = vn;
+    }
+    if constexpr (!EXACT) {
+        // The flagged elements again, operation by operation.  A wavefront with no flagged element branches past
+        // this; otherwise only the element positions that are flagged in some lane are redone.
+        if (__builtin_amdgcn_ballot_w64(any_redo) != 0) {
+#pragma unroll
+            for (int k = 0; k < EPL; ++k) {
+                if (__builtin_amdgcn_ballot_w64(redo[k]) != 0) {
+                    float pk = master_of<DT, ECCB, EPL>(raw.p, raw.e, k, lut);
+                    if constexpr (DECOUPLED) pk = pk * h.one_m_wd;
+                    const float pe = adam_apply_exact(pk, m[k], v[k], h);
+                    if (redo[k]) p[k] = pe;
+                }
+            }
+        }
     }
 
     Pack<ECCB, EPL> eout;
@@ -84,27 +101,17 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
 #pragma unroll
         for (int k = 0; k < EPL; k += 2) {  // pairs, so that each step is one three-operand max
             am = fmaxf(fmaxf(am, fabsf(m[k])), fabsf(m[k + 1]));
-            if constexpr (MAY_BE_QUICK) av = fmaxf(fmaxf(av, v[k]), v[k + 1]);
-            else av = fmaxf(fmaxf(av, r[k]), r[k + 1]);
+            av = fmaxf(fmaxf(av, v[k]), v[k + 1]);
         }
         am = fmaxf(group_max<EPL>(am), 1e-12f);
-        av = group_max<EPL>(av);
-        if constexpr (MAY_BE_QUICK) {
-            const float av_quick = fmaxf(hw::sqrt(av), 1e-12f);   // av holds the group's largest v here
-            av = fmaxf(sqrt_corrected(av), 1e-12f);               // what the exact requantiser divides by, and the scale
-            if constexpr (EPL == 8) {
-                quantize_mom_quick_verified<EPL>(m, am, raw.m);
-                quantize_var_quick_verified<EPL>(v, r, av_quick, av, raw.v);
-            } else {
-                quantize_mom_var_quick_verified(m, am, v, r, av_quick, av, raw.m, raw.v);
-            }
-        } else if constexpr (EPL == 8) {
-            av = fmaxf(av, 1e-12f);
-            quantize_mom<EPL>(m, am, raw.m);
-            quantize_var<EPL>(r, av, raw.v);
+        av = group_max<EPL>(av);                              // the group's largest v
+        const float av_quick = fmaxf(hw::sqrt(av), 1e-12f);
+        av = fmaxf(sqrt_corrected(av), 1e-12f);               // what the exact requantiser divides by, and the scale
+        if constexpr (EPL == 8) {
+            quantize_mom_quick_verified<EPL>(m, am, raw.m);
+            quantize_var_quick_verified<EPL>(v, r, av_quick, av, raw.v);
         } else {
-            av = fmaxf(av, 1e-12f);
-            quantize_mom_var(m, am, r, av, raw.m, raw.v);
+            quantize_mom_var_quick_verified(m, am, v, r, av_quick, av, raw.m, raw.v);
         }
         store_lane<1, EPL, FAST>(raw.m, t.mom, w, n);
         store_lane<1, EPL, FAST>(raw.v, t.var, w, n);
@@ -200,8 +207,10 @@ template <int DT, int EB, bool Q> using AdamWOp = fo::AdamOp<DT, EB, Q, true>;  
 template <int DT, int EB, bool Q> using AdamL2ExactOp = fo::AdamOp<DT, EB, Q, false, true>;
 template <int DT, int EB, bool Q> using AdamWExactOp = fo::AdamOp<DT, EB, Q, true, true>;
 
+// exact: the caller asked for the operation-by-operation update on every element; a launch whose folded constants
+// are out of range (fo_math.h: make_adam_hyper) takes it too.
 template <class L> int dispatch_adam(int dtype, int ecc_bytes, int quantized, int decoupled, int exact, L&& launcher) {
-    if (exact)
+    if (exact || !launcher.h.folded_ok)
         return decoupled ? dispatch<AdamWExactOp>(dtype, ecc_bytes, quantized, launcher)
                          : dispatch<AdamL2ExactOp>(dtype, ecc_bytes, quantized, launcher);
     return decoupled ? dispatch<AdamWOp>(dtype, ecc_bytes, quantized, launcher) : dispatch<AdamL2Op>(dtype, ecc_bytes, quantized, launcher);
@@ -382,7 +391,7 @@ int fo_multi_adam_step_static(const fo_tensor_desc* host_descs, int64_t n_tensor
         if (int rc = check_hip(hipGetLastError(), "table staging kernel launch")) return rc;
     }
     MultiLauncher<fo::AdamHyper> L{d_descs, d_chunks, n_chunks, make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step), (hipStream_t)stream};
-    return decoupled ? dispatch<AdamWOp>(dtype, ecc_bytes, quantized, L) : dispatch<AdamL2Op>(dtype, ecc_bytes, quantized, L);
+    return dispatch_adam(dtype, ecc_bytes, quantized, decoupled, 0, L);
 }
 
 int fo_multi_adam_streams_copy(const fo_tensor_desc* descs, int64_t n_tensors, const fo_chunk* chunks, int64_t n_chunks,

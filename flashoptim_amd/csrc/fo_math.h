@@ -115,6 +115,16 @@ FO_FN float sqrt_corrected(float x) {
     return hw::fma(rem, h, s);
 }
 
+// RN(q / 255) for an integer q in 0..255 (ref:2333): the product with 1/255 held as a two-term constant,
+// fma(q, k_hi, q * k_lo) with k_hi + k_lo = 1/255 to 2^-50.  The correctly rounded quotient for each of the 256
+// codes (checked exhaustively on the host); q * RN(1/255) alone misses it for 126 of them.
+FO_FN float code_over_255(float q) {
+    constexpr double k = 1.0 / 255.0;
+    constexpr float k_hi = (float)k;
+    constexpr float k_lo = (float)(k - (double)k_hi);
+    return hw::fma(q, k_hi, q * k_lo);
+}
+
 // ------------------------------------------------------------------------------------------------
 // ECC: narrow value + signed integer fraction of half its ulp (ref:2682-2776)
 // ------------------------------------------------------------------------------------------------
@@ -278,7 +288,9 @@ struct AdamHyper {
     //     lr * (m / bc1) / (sqrt(v / bc2) + eps)  ==  m / (sqrt(v) * den_scale + den_bias)
     //     den_scale = bc1 / (lr * sqrt(bc2)),  den_bias = eps * bc1 / lr
     float neg_den_scale, neg_den_bias;
-    float sqrt_b2_over_255;  // dequantised sqrt(v_old * b2) = code * scale * sqrt(b2) / 255
+    // host only: the folded constants are ordinary numbers (see make_adam_hyper); otherwise the launch takes the
+    // operation-by-operation kernel
+    int folded_ok;
     // operation-by-operation form (EXACT): the reference's own sequence with correctly rounded quotients
     float lr, eps, bc1, rcp_bc1, bc2, rcp_bc2;  // rcp_*: correctly rounded reciprocals, formed on the host
 };
@@ -289,7 +301,6 @@ inline AdamHyper make_adam_hyper(float lr, float beta1, float beta2, float eps, 
     h.b1 = beta1; h.one_m_b1 = 1.0f - beta1;
     h.b2 = beta2; h.one_m_b2 = 1.0f - beta2;
     h.wd = wd; h.one_m_wd = 1.0f - wd;
-    h.sqrt_b2_over_255 = (float)(std::sqrt((double)beta2) / 255.0);
     // beta^step is the correctly rounded fp32 power, 1 - that is formed in fp32 (ref:2368-2369)
     h.bc1 = 1.0f - (float)std::pow((double)beta1, (double)step);
     h.bc2 = 1.0f - (float)std::pow((double)beta2, (double)step);
@@ -304,43 +315,37 @@ inline AdamHyper make_adam_hyper(float lr, float beta1, float beta2, float eps, 
         h.neg_den_scale = 0.0f;
         h.neg_den_bias = -std::numeric_limits<float>::infinity();
     }
+    // The folded update's error bound (adam_apply_folded) assumes that both constants carry a full fp32 mantissa and
+    // that sqrt(v) * den_scale neither overflows nor turns subnormal for any fp32 v: den_scale within 2^-40 .. 2^60
+    // (lr between about 1e-18 and 1e12) and den_bias zero or a normal number.  lr == 0 is exact as it stands.
+    const double ds = std::fabs((double)h.neg_den_scale), db = std::fabs((double)h.neg_den_bias);
+    h.folded_ok = lr == 0.0f || (lr > 0.0f && ds >= 0x1p-40 && ds <= 0x1p60 && (db == 0.0 || (db >= 0x1p-126 && db <= 0x1p100)));
     return h;
 }
 
-// Which variants follow the reference's update operation by operation (EXACT) instead of the folded form:
-// fp32 parameters, where one fp32 ulp is the master precision and the 16.25 bytes per element leave room
-// for the extra arithmetic.  Narrow parameters use the folded update (see adam_apply).
-template <int DT, int ECCB> struct AdamExact { static constexpr bool value = DT == DT_F32; };
-// Variants that form the new moments with the decay folded into the group scale (adam_moments_quantized): bf16
-// parameters.  fp16 parameters keep the reference's operation order for the moments although their update is
-// folded: fp16 gradients underflow into a handful of subnormal values, moments built from so few distinct values
-// sit exactly on rounding boundaries in bulk, and the folded form's one-ulp differences then move up to 1e-2 of
-// the codes; with the unfolded moments and the exact requantiser their codes and scales equal the oracle's always.
-template <int DT, int ECCB> struct AdamFoldedMoments { static constexpr bool value = DT == DT_BF16; };
+// Which variants follow the reference's update operation by operation on every element (EXACT): those whose unit
+// of master precision is about one fp32 ulp or finer, so that nothing but the reference's own sequence of
+// roundings meets it -- fp32 parameters, 2-byte parameters with a 2-byte ECC (32-bit masters: the unit is
+// 32768/32767 fp32 ulps), fp16 parameters with a 1-byte ECC (unit 2^-19 of the weight).  bf16 parameters with a
+// 1-byte ECC (24-bit masters, unit 2^-16 of the weight) and 2-byte parameters without ECC (unit = one ulp of the
+// narrow type) take the folded update and redo operation by operation only the elements it cannot vouch for
+// (adam_apply_folded below).
+template <int DT, int ECCB> struct AdamExact {
+    static constexpr bool value = DT == DT_F32 || ECCB == 2 || (DT == DT_F16 && ECCB == 1);
+};
 // Variants that use the quick requantiser forms (verified value by value, see above; the codes are the exact
-// forms' either way): all but the folded update with a 2-byte ECC, whose 14.25 bytes per element hide the exact
-// requantiser's arithmetic (measured: no gain).  The operation-by-operation update uses them with any ECC width.
-template <int DT, int ECCB> struct AdamQuickRequant { static constexpr bool value = DT == DT_F32 || ECCB != 2; };
+// forms' either way): every one.
+template <int DT, int ECCB> struct AdamQuickRequant { static constexpr bool value = true; };
 
-// New moments from the dequantised pieces.
-//   EXACT = false: the EMA decay is folded into the group scale (one multiply per lane instead of one per
-//   element): m = fma(table[qm], sm * b1, g * (1 - b1)); v = fma(s, s, g^2 * (1 - b2)), s = qv * sv * sqrt(b2)/255.
-//   From an all-zero state both equal the reference's values bit for bit.
-//   EXACT = true: every operation of ref:2332-2360 rounded on its own.
-template <bool EXACT>
-FO_FN void adam_moments_quantized(float g, float table_m, float sm, float sm_b1, float qv, float sv, float sv_b2,
-                                  const AdamHyper& h, float& mn, float& vn) {
-    if constexpr (EXACT) {
-        const float mo = table_m * sm;                                              // ref:2332-2343
-        const float s = div_corrected(qv, 255.0f, 1.0f / 255.0f) * sv;               // ref:2333-2347
-        const float vo = s * s;                                                     // ref:2348
-        mn = mo * h.b1 + g * h.one_m_b1;                                            // ref:2357
-        vn = vo * h.b2 + (g * g) * h.one_m_b2;                                      // ref:2360
-    } else {
-        mn = hw::fma(table_m, sm_b1, g * h.one_m_b1);
-        const float s = qv * sv_b2;
-        vn = hw::fma(s, s, (g * g) * h.one_m_b2);
-    }
+// New moments from the dequantised pieces, every operation of ref:2332-2360 rounded on its own.
+//   table_m: (q/127) / (2 - |q/127|) of the first-moment code (StepTables); qv: the second-moment code as a float.
+FO_FN void adam_moments_quantized(float g, float table_m, float sm, float qv, float sv, const AdamHyper& h, float& mn,
+                                  float& vn) {
+    const float mo = table_m * sm;                                              // ref:2332-2343
+    const float s = code_over_255(qv) * sv;                                     // ref:2333-2347
+    const float vo = s * s;                                                     // ref:2348
+    mn = mo * h.b1 + g * h.one_m_b1;                                            // ref:2357
+    vn = vo * h.b2 + (g * g) * h.one_m_b2;                                      // ref:2360
 }
 // Unquantised states: operation by operation as written in the reference, no contraction (ref:2351-2360).
 FO_FN void adam_moments_plain(float g, float mo, float vo, const AdamHyper& h, float& mn, float& vn) {
@@ -348,19 +353,48 @@ FO_FN void adam_moments_plain(float g, float mo, float vo, const AdamHyper& h, f
     vn = vo * h.b2 + (g * g) * h.one_m_b2;
 }
 
-// p -= lr * (m/bc1) / (sqrt(v/bc2) + eps)  (ref:2368-2375).  r = sqrt(v), shared with the requantiser.
-template <bool EXACT> FO_FN float adam_apply(float p, float mn, float vn, float r, const AdamHyper& h) {
-    if constexpr (EXACT) {
-        const float cm = div_corrected(mn, h.bc1, h.rcp_bc1);
-        const float cv = div_corrected(vn, h.bc2, h.rcp_bc2);
-        const float den = sqrt_corrected(cv) + h.eps;
-        float rd = hw::rcp(den);
-        rd = hw::fma(hw::fma(-den, rd, 1.0f), rd, rd);  // reciprocal refined to well below an ulp
-        return p - div_corrected(h.lr * cm, den, rd);
-    } else {
-        const float neg_den = hw::fma(r, h.neg_den_scale, h.neg_den_bias);
-        return hw::fma(mn, hw::rcp(neg_den), p);
-    }
+// p -= lr * (m/bc1) / (sqrt(v/bc2) + eps), operation by operation (ref:2368-2375): every quotient and the root
+// correctly rounded.  p: the weight after the decoupled decay, if any.
+FO_FN float adam_apply_exact(float p, float mn, float vn, const AdamHyper& h) {
+    const float cm = div_corrected(mn, h.bc1, h.rcp_bc1);
+    const float cv = div_corrected(vn, h.bc2, h.rcp_bc2);
+    const float den = sqrt_corrected(cv) + h.eps;
+    float rd = hw::rcp(den);
+    rd = hw::fma(hw::fma(-den, rd, 1.0f), rd, rd);  // reciprocal refined to well below an ulp
+    return p - div_corrected(h.lr * cm, den, rd);
+}
+
+// The folded update and its guard.
+//   Folded: u = m * rcp(-(r c1 + c2)) with r = hw::sqrt(v) and c1, c2 the host-folded constants (AdamHyper), then
+//   p_new = fma(p, 1 - wd, u) (decoupled decay) or p + u: four instructions, where the reference's sequence costs
+//   about twenty.  With u = 2^-24 (half an ulp, relative) the two evaluations of the update differ by at most
+//       reference   lr*cm: 2u;  cv: u -> root u/2, rounding of the root u, of the sum with eps u;  quotient u    = 5.5u
+//       folded      r: one ulp = 2u, c1: u, fma: u, rcp: one ulp = 2u, product: u                                = 7u
+//   i.e. by 12.5u |update| from identical m and v (the moments are formed operation by operation in both), and
+//   the fused decay rounds p(1 - wd) once less than the reference: u |p(1 - wd)| <= u (|p_new| + |update|).  With
+//   the final rounding of either side (u |p_new| each) the two fp32 results are at most
+//       13.5u |update| + 3u |p_new|
+//   apart.  They are split into the same narrow value and a correction code that differs by at most one -- the
+//   master weights agree to within one unit of master precision -- whenever that distance is below one unit,
+//   and a unit is at least G |p_new| with G = 2^-16 for bf16 + 1-byte ECC (2^(E-8)/127 against |p_new| <
+//   2^(E+1)), 2^-8 for bf16 without ECC (one bf16 ulp) and 2^-11 for fp16 without ECC:
+//       13.5u |update| < (G - 3u) |p_new|   <=>   |update| < (2^24 G - 3) / 13.5 |p_new|
+//   = 18.7, 4854 and 606 times |p_new|.  kGuard is the power of two below (16, 4096, 512); an element whose
+//   folded update exceeds kGuard |p_new| -- a weight that its own update all but cancels: 1e-3 of the elements on a
+//   first step with weights ~N(0, 0.02) and lr 1e-3, fewer later -- is flagged and the caller redoes it with
+//   adam_apply_exact, whose result is the reference's bit for bit.  Every other element is within one unit by
+//   the bound above, whatever the data.
+template <int DT, int ECCB> struct AdamFoldedGuard {
+    static_assert(!AdamExact<DT, ECCB>::value, "the folded update is not offered for this variant");
+    static constexpr float value = ECCB == 1 ? 16.0f : (DT == DT_BF16 ? 4096.0f : 512.0f);
+};
+template <bool DECOUPLED>
+FO_FN float adam_apply_folded(float p, float mn, float r, const AdamHyper& h, float guard, bool& redo) {
+    const float neg_den = hw::fma(r, h.neg_den_scale, h.neg_den_bias);
+    const float u = mn * hw::rcp(neg_den);
+    const float pn = DECOUPLED ? hw::fma(p, h.one_m_wd, u) : p + u;
+    redo = fabsf(pn) * guard < fabsf(u);
+    return pn;
 }
 
 // ------------------------------------------------------------------------------------------------

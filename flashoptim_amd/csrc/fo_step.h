@@ -52,19 +52,24 @@ __device__ __forceinline__ bool all_aligned16(const TensorPtrs& t) {
 // shared pieces of the step kernels
 // ------------------------------------------------------------------------------------------------
 
-// Reads the lane's parameter values as fp32 masters (ref:2299-2309).
+// One parameter value as an fp32 master (ref:2299-2309).
 // An int8 ECC byte goes through the LDS table of correctly rounded fractions (one lookup instead of a convert and
 // two multiply-adds); int16 codes are converted arithmetically.
+template <int DT, int ECCB, int EPL>
+__device__ __forceinline__ float master_of(const Pack<DTypeInfo<DT>::bytes, EPL>& praw, const Pack<ECCB, EPL>& eraw, int k,
+                                           const float* lut) {
+    const float w = widen<DT, EPL>(praw, k);
+    if constexpr (ECCB == 1) return ecc_join_fraction<DT>(w, lookup_ecc(lut, byte_of<EPL>(eraw, k)));
+    else if constexpr (ECCB == 2) return ecc_join<DT, ECCB>(w, ecc_to_float<ECCB, EPL>(eraw, k));
+    else return w;
+}
+
+// The lane's parameter values as fp32 masters.
 template <int DT, int ECCB, int EPL>
 __device__ __forceinline__ void read_master(float (&p)[EPL], const Pack<DTypeInfo<DT>::bytes, EPL>& praw,
                                             const Pack<ECCB, EPL>& eraw, const float* lut) {
 #pragma unroll
-    for (int k = 0; k < EPL; ++k) {
-        const float w = widen<DT, EPL>(praw, k);
-        if constexpr (ECCB == 1) p[k] = ecc_join_fraction<DT>(w, lookup_ecc(lut, byte_of<EPL>(eraw, k)));
-        else if constexpr (ECCB == 2) p[k] = ecc_join<DT, ECCB>(w, ecc_to_float<ECCB, EPL>(eraw, k));
-        else p[k] = w;
-    }
+    for (int k = 0; k < EPL; ++k) p[k] = master_of<DT, ECCB, EPL>(praw, eraw, k, lut);
 }
 
 // Narrows the updated masters and derives the new ECC (ref:2377-2387).
@@ -84,34 +89,6 @@ __device__ __forceinline__ void write_master(const float (&p)[EPL], Pack<DTypeIn
     if constexpr (ECCB > 0) pack_codes<ECCB, EPL>(eb, eout);
 }
 
-// Quantises the lane's first-moment values against the group absmax `am` (shared by the group's lanes, clamped
-// at 1e-12) and the lane's sqrt(v) values against the group maximum `av`; the rounding is the reference's
-// (fo_math.h: quantize_mom_rounded, quantize_var_rounded; ref:2405-2419, 1703-1710).
-template <int EPL>
-__device__ __forceinline__ void quantize_mom(const float (&m)[EPL], float am, Pack<1, EPL>& out) {
-    static_assert(EPL == 8, "two dwords of codes per lane");
-    const float ram = hw::rcp(am);
-    float lo[4], hi[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        lo[k] = quantize_mom_rounded(m[k], am, ram);
-        hi[k] = quantize_mom_rounded(m[k + 4], am, ram);
-    }
-    convert_pack8<kFloor, kFloor>(lo, hi, out.w[0], out.w[1]);
-}
-template <int EPL>
-__device__ __forceinline__ void quantize_var(const float (&r)[EPL], float av, Pack<1, EPL>& out) {
-    static_assert(EPL == 8, "two dwords of codes per lane");
-    const float rav = hw::rcp(av);
-    float lo[4], hi[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        lo[k] = quantize_var_rounded(r[k], av, rav);
-        hi[k] = quantize_var_rounded(r[k + 4], av, rav);
-    }
-    convert_pack8<kTrunc, kTrunc>(lo, hi, out.w[0], out.w[1]);
-}
-
 // Replaces byte k of the lane's packed codes.
 template <int EPL> __device__ __forceinline__ void set_code(Pack<1, EPL>& out, int k, u32 code) {
     const int sh = 8 * (k & 3);
@@ -119,8 +96,9 @@ template <int EPL> __device__ __forceinline__ void set_code(Pack<1, EPL>& out, i
     w = (w & ~(0xffu << sh)) | ((code & 0xffu) << sh);
 }
 
-// The same through the quick forms (fo_math.h): every value is converted from its quick form; the values that
-// fail the margin test are redone with the exact form.  A wavefront with no failing value (about four in five on
+// Quantises the lane's first-moment values against the group absmax `am` (shared by the group's lanes, clamped
+// at 1e-12); the rounding is the reference's (fo_math.h; ref:2405-2419, 1703-1710).  Through the quick forms:
+// every value is converted from its quick form; the values that fail the margin test are redone with the exact form.  A wavefront with no failing value (about four in five on
 // continuous data) branches past the repair; otherwise only the element positions k that failed in some lane are
 // redone.  The result is the exact requantiser's, code for code.
 template <int EPL>
@@ -208,18 +186,6 @@ __device__ __forceinline__ void quantize_mom_var_quick_verified(const float (&m)
             }
         }
     }
-}
-// Four elements per lane (fp32 parameters): one dword of codes per state; the two states share the conversion block.
-__device__ __forceinline__ void quantize_mom_var(const float (&m)[4], float am, const float (&r)[4], float av,
-                                                 Pack<1, 4>& mout, Pack<1, 4>& vout) {
-    const float ram = hw::rcp(am), rav = hw::rcp(av);
-    float a[4], b[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        a[k] = quantize_mom_rounded(m[k], am, ram);
-        b[k] = quantize_var_rounded(r[k], av, rav);
-    }
-    convert_pack8<kFloor, kTrunc>(a, b, mout.w[0], vout.w[0]);
 }
 // Four elements per lane, one state (momentum kernels on fp32 parameters): plain conversion and byte packing.
 __device__ __forceinline__ void quantize_mom(const float (&m)[4], float am, Pack<1, 4>& out) {
@@ -354,38 +320,58 @@ inline int validate_multi(const fo_tensor_desc* descs, int64_t n_tensors, const 
 // Streaming from HBM degrades when a compute unit keeps too many bytes in flight, and a step wavefront has
 // several KiB of loads outstanding.  Each kernel family therefore names the number of workgroups it wants
 // resident per compute unit (Op::kWorkgroupsPerCu, the best of those measured on MI355X) and the launch requests
-// enough unused dynamic LDS to cap the residency there.  gfx950 hands out LDS in units of 320 dwords, 128 of them
-// per compute unit, so the counts that can be reached this way are 128 / k: ... 12, 14, 16, 18, 21, 25, 32 (measured
-// durations fall on exactly these plateaus, whatever finer count the runtime's occupancy query grants).  A family
-// may also cap the wavefronts per SIMD (Op::kMaxWavesPerSimd); the query reports the smaller of the two limits.
+// enough unused dynamic LDS to cap the residency there.  MI355X hands out its 160 KiB of LDS per compute unit in 128
+// units of 320 dwords, so the counts that can be reached this way are 128 / k: ... 12, 14, 16, 18, 21, 25, 32
+// (measured durations fall on exactly these plateaus, whatever finer count the runtime's occupancy query grants).
+// The allocation unit is not something the runtime reports: on a device whose LDS per compute unit is not those
+// 160 KiB the plan does not assume it and sizes the request from the occupancy query alone (lds / target bytes).
+// A family may also cap the wavefronts per SIMD (Op::kMaxWavesPerSimd: the kernel descriptor then declares enough
+// registers that a SIMD holds no more; the occupancy query does not see that padding, so the cap is applied here).
 struct Residency {
     int target = 0;    // workgroups per compute unit asked for
-    int achieved = 0;  // what the LDS units and the occupancy query allow with `dynamic_lds`
+    int achieved = 0;  // what the LDS request, the occupancy query and the cap per SIMD allow together
     unsigned dynamic_lds = 0;
+    int lds_unit_bytes = 0;  // allocation unit assumed (0: unknown device, the occupancy query alone was used)
 };
 
-constexpr long kLdsUnitBytes = 1280;
+constexpr long kLdsUnitBytes = 1280;     // MI355X: 320 dwords
+constexpr long kLdsUnitsPerCu = 128;     // 160 KiB / 1280
+constexpr int kSimdsPerCu = 4;
 
 template <class Kernel>
-Residency plan_residency(Kernel kernel, int target, int static_lds) {
+Residency plan_residency(Kernel kernel, int target, int static_lds, int max_waves_per_simd) {
     Residency r;
     r.target = target;
     int dev = 0, lds_per_cu = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&lds_per_cu, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, dev) != hipSuccess || lds_per_cu <= 0)
         return r;
-    // the most LDS units per workgroup that still admit `target` workgroups
-    const long units_per_cu = lds_per_cu / kLdsUnitBytes;
-    long units = units_per_cu / target;
-    const long least = (static_lds + kLdsUnitBytes - 1) / kLdsUnitBytes;
-    if (units < least) units = least;
-    if (units < 1) units = 1;
-    const long bytes = units * kLdsUnitBytes;
+    // one launch may ask for at most 64 KiB of LDS: fewer than three workgroups per compute unit cannot be enforced
+    constexpr long kMaxLdsPerLaunch = 65536;
+    long bytes, by_units;
+    if (lds_per_cu == kLdsUnitBytes * kLdsUnitsPerCu) {
+        // the most LDS units per workgroup that still admit `target` workgroups
+        long units = kLdsUnitsPerCu / target;
+        const long least = (static_lds + kLdsUnitBytes - 1) / kLdsUnitBytes;
+        if (units < least) units = least;
+        if (units < 1) units = 1;
+        if (units * kLdsUnitBytes > kMaxLdsPerLaunch) units = kMaxLdsPerLaunch / kLdsUnitBytes;
+        bytes = units * kLdsUnitBytes;
+        by_units = kLdsUnitsPerCu / units;
+        r.lds_unit_bytes = (int)kLdsUnitBytes;
+    } else {
+        bytes = (lds_per_cu / target) & ~255L;
+        if (bytes > kMaxLdsPerLaunch) bytes = kMaxLdsPerLaunch;
+        if (bytes < static_lds) bytes = static_lds;
+        by_units = INT32_MAX;  // unknown unit: trust the query
+    }
     const long dyn = bytes > static_lds ? bytes - static_lds : 0;
     int granted = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&granted, kernel, fo::kBlockThreads, (size_t)dyn) != hipSuccess) granted = 0;
-    const long by_units = units_per_cu / units;
-    r.achieved = granted < by_units ? granted : (int)by_units;
+    long achieved = granted < by_units ? granted : by_units;
+    const long by_simd = (long)kSimdsPerCu * max_waves_per_simd;
+    if (achieved > by_simd) achieved = by_simd;
+    r.achieved = (int)achieved;
     r.dynamic_lds = (unsigned)dyn;
     return r;
 }
@@ -400,7 +386,7 @@ template <class Op, class Kernel> const Residency& residency_of(Kernel kernel) {
     std::call_once(once[dev], [&] {
         const int forced = debug_workgroups_per_cu();
         constexpr int kStatic = fo::StepLut<Op::kLutTables>::kFloats * 4;
-        cache[dev] = plan_residency(kernel, forced > 0 ? forced : Op::kWorkgroupsPerCu, kStatic);
+        cache[dev] = plan_residency(kernel, forced > 0 ? forced : Op::kWorkgroupsPerCu, kStatic, Op::kMaxWavesPerSimd);
     });
     return cache[dev];
 }

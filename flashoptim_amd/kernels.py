@@ -266,9 +266,10 @@ def _fused_adam_step(
     """One fused Adam/AdamW step on one contiguous tensor (ref:2203-2251).  ``weight_decay`` is already
     multiplied by lr (or lr/initial_lr) for the decoupled optimizers.
 
-    ``exact_update`` (not in the reference): evaluate the update operation by operation as the reference writes it,
-    for bf16 / fp16 parameters too (fp32 parameters always are); every output bit then equals an IEEE evaluation of
-    the reference's formulas, at 5-11 % less throughput."""
+    ``exact_update`` (not in the reference): evaluate the update operation by operation as the reference writes it
+    on every element of every variant; every output bit then equals an IEEE evaluation of the reference's formulas.
+    The default already does so except for bf16 parameters with an int8 correction term and 2-byte parameters
+    without one, whose folded update keeps every master weight within one unit of master precision."""
     _check_group_size(group_size)
     n = param.numel()
     if n == 0:

@@ -140,13 +140,16 @@ int fo_multi_adam_step_static(const fo_tensor_desc *host_descs, int64_t n_tensor
 /*
  * fo_adam_step / fo_multi_adam_step with the update evaluated operation by operation as the reference writes it,
  *     p -= (lr * (m / bc1)) / (sqrt(v / bc2) + eps)          (ref:2368-2375)
- * with correctly rounded quotients and roots and the moments formed without folding (ref:2332-2360), for every
- * parameter dtype.  Every output bit then equals an IEEE evaluation of the reference's formulas.  The plain entry
- * points do this for fp32 parameters only; for bf16 / fp16 parameters they fold the bias corrections and the
- * learning rate into two constants (one reciprocal per element), which leaves 1e-4 (24-bit masters) to 2e-2
- * (32-bit masters) of the master weights more than one unit of master precision away from that evaluation, and is
- * roughly 5-12 % faster.  Same arguments and errors as the plain entry points.  The reference has one kernel and no such
- * choice; these are for callers who want the stricter arithmetic.
+ * with correctly rounded quotients and roots, on every element and for every parameter dtype: every output bit
+ * then equals an IEEE evaluation of the reference's formulas.
+ * The plain entry points already do this wherever nothing else meets one unit of master precision: fp32
+ * parameters, 2-byte parameters with a 2-byte ECC (32-bit masters), fp16 parameters with a 1-byte ECC.  For bf16
+ * parameters with a 1-byte ECC (24-bit masters) and 2-byte parameters without ECC they fold the bias corrections
+ * and the learning rate into two constants (one reciprocal per element) and redo operation by operation only the
+ * elements whose update all but cancels the weight; moment codes and scales are then still bit-identical and
+ * every master weight lies within one unit of master precision, but the correction code may differ by one step.
+ * Same arguments and errors as the plain entry points.  The reference has one kernel and no such choice; these
+ * are for callers who want every bit.
  */
 int fo_adam_step_exact(void *mom, void *mom_scales, void *var, void *var_scales, void *param, const void *grad,
                        void *ecc, int64_t n, int dtype, int ecc_bytes, int quantized, float lr, float beta1,

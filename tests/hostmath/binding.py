@@ -37,7 +37,11 @@ def lib() -> ctypes.CDLL:
         vp, i64, i32, f = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
         L.hm_set_noise.argtypes = [i32]
         L.hm_set_noise.restype = None
-        L.hm_adam_step.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, f, f, f, f, f, i32, i32, i32]
+        L.hm_adam_step.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, f, f, f, f, f, i32, i32, i32, ctypes.POINTER(i64)]
+        L.hm_adam_folded_update.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, f, f, f, f, f, i32, i32, vp, vp]
+        L.hm_adam_folded_update.restype = None
+        L.hm_code_over_255.argtypes = [vp]
+        L.hm_code_over_255.restype = None
         L.hm_momentum_step.argtypes = [vp, vp, vp, vp, vp, i64, i32, i32, i32, f, f, f, f, i32, i32, i32]
         L.hm_sgd_plain_step.argtypes = [vp, vp, vp, i64, i32, i32, f, f, i32]
         L.hm_div_corrected.argtypes = [vp, vp, vp, i64]
@@ -75,11 +79,36 @@ def _ecc_bytes(ecc) -> int:
 
 
 def adam_step(mom, mom_scales, var, var_scales, param, grad, ecc, lr, beta1, beta2, eps, weight_decay, decoupled, step,
-              quantized: bool = True, exact: int = -1) -> None:
+              quantized: bool = True, exact: int = -1) -> int:
+    """One Adam step as the kernels compute it.  exact <= 0: what fo_adam_step does for this variant; 1: the
+    operation-by-operation update on every element (fo_adam_step_exact).  Returns the number of elements whose
+    folded update the guard sent through the operation-by-operation form."""
+    flagged = ctypes.c_int64(0)
     rc = lib().hm_adam_step(_ptr(mom), _ptr(mom_scales), _ptr(var), _ptr(var_scales), _ptr(param), _ptr(grad), _ptr(ecc),
                             param.numel(), _DTYPE_CODE[param.dtype], _ecc_bytes(ecc), int(quantized), lr, beta1, beta2,
-                            eps, weight_decay, int(decoupled), int(step), int(exact))
+                            eps, weight_decay, int(decoupled), int(step), int(exact), ctypes.byref(flagged))
     assert rc == 0
+    return int(flagged.value)
+
+
+def adam_folded_update(param, ecc, grad, mom, mom_scales, var, var_scales, lr, beta1, beta2, eps, weight_decay, decoupled, step):
+    """The folded Adam update of bf16 parameters with an int8 ECC and quantised states without the repair of the
+    flagged elements.  Returns (fp32 results, bool tensor of the elements the guard flags); nothing is changed in
+    place."""
+    assert param.dtype == torch.bfloat16 and ecc.dtype == torch.int8
+    n = param.numel()
+    out = torch.empty(n, dtype=torch.float32)
+    redo = torch.empty(n, dtype=torch.uint8)
+    lib().hm_adam_folded_update(_ptr(mom), _ptr(mom_scales), _ptr(var), _ptr(var_scales), _ptr(param), _ptr(grad), _ptr(ecc), n,
+                                lr, beta1, beta2, eps, weight_decay, int(decoupled), int(step), out.data_ptr(), redo.data_ptr())
+    return out, redo.bool()
+
+
+def code_over_255() -> torch.Tensor:
+    """code_over_255(q) of fo_math.h for q = 0 .. 255."""
+    out = torch.empty(256, dtype=torch.float32)
+    lib().hm_code_over_255(out.data_ptr())
+    return out
 
 
 def momentum_step(mom, scales, param, grad, ecc, lr, mom_coef, update_coef, weight_decay, decoupled=False, nesterov=False,

@@ -81,57 +81,53 @@ template <int DT, int ECCB> void write_master(void* param, void* ecc, int64_t i,
     if constexpr (ECCB > 0) store_ecc<ECCB>(ecc, i, ecc_split_bits<DT, ECCB, false>(p, w));
 }
 
-// the structure of adam_finish (fo_adam.hip), one quantisation group at a time
+// the structure of adam_finish (fo_adam.hip), one quantisation group at a time.  `flagged` (may be null) counts the
+// elements whose folded update was redone operation by operation.
 template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT>
 void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scales, void* param, const void* grad, void* ecc,
-                 int64_t n, const AdamHyper& h) {
-    constexpr bool kQuick = QUANT && (AdamQuickRequant<DT, ECCB>::value || EXACT);
-    constexpr bool kExactMoments = EXACT || !AdamFoldedMoments<DT, ECCB>::value;
+                 int64_t n, const AdamHyper& h, int64_t* flagged) {
     for (int64_t g0 = 0; g0 < n; g0 += kGroup) {
         const int cnt = (int)((n - g0) < kGroup ? (n - g0) : kGroup);
         const int64_t group = g0 >> 5;
         float sm = 1.0f, sv = 1.0f;
         if (QUANT) { sm = f16_to_f32(mom_scales[group]); sv = f16_to_f32(var_scales[group]); }
-        const float sm_b1 = sm * h.b1, sv_b2 = sv * h.sqrt_b2_over_255;
-        float m[kGroup], r[kGroup], v[kGroup];
-        float am = 0.0f, av = 0.0f, vmax = 0.0f;
+        float m[kGroup], v[kGroup];
+        float am = 0.0f, vmax = 0.0f;
         for (int k = 0; k < cnt; ++k) {
             const int64_t i = g0 + k;
-            float p = read_master<DT, ECCB>(param, ecc, i);
+            const float p0 = read_master<DT, ECCB>(param, ecc, i);
             float gr = load_elem<DT>(grad, i);
-            if (!DECOUPLED) gr = gr + p * h.wd;
+            if (!DECOUPLED) gr = gr + p0 * h.wd;
             float mn, vn;
             if (QUANT) {
-                adam_moments_quantized<kExactMoments>(gr, kTable.v[((const uint8_t*)mom)[i]], sm, sm_b1,
-                                                      (float)((const uint8_t*)var)[i], sv, sv_b2, h, mn, vn);
+                adam_moments_quantized(gr, kTable.v[((const uint8_t*)mom)[i]], sm, (float)((const uint8_t*)var)[i], sv, h, mn, vn);
             } else {
                 adam_moments_plain(gr, load_elem<DT>(mom, i), load_elem<DT>(var, i), h, mn, vn);
             }
-            if (DECOUPLED) p = p * h.one_m_wd;
-            const float rk = (QUANT || !EXACT) ? (kQuick ? hw::sqrt(vn) : sqrt_corrected(vn)) : 0.0f;
-            p = adam_apply<EXACT>(p, mn, vn, rk, h);
+            float p;
+            if constexpr (EXACT) {
+                p = adam_apply_exact(DECOUPLED ? p0 * h.one_m_wd : p0, mn, vn, h);
+            } else {
+                bool redo;
+                p = adam_apply_folded<DECOUPLED>(p0, mn, hw::sqrt(vn), h, AdamFoldedGuard<DT, ECCB>::value, redo);
+                if (redo) {
+                    p = adam_apply_exact(DECOUPLED ? p0 * h.one_m_wd : p0, mn, vn, h);
+                    if (flagged) ++*flagged;
+                }
+            }
             write_master<DT, ECCB>(param, ecc, i, p);
-            m[k] = mn; r[k] = rk; v[k] = vn;
+            m[k] = mn; v[k] = vn;
             am = fmaxf(am, fabsf(mn));
-            av = fmaxf(av, rk);
             vmax = fmaxf(vmax, vn);
         }
         if (QUANT) {
+            // quick forms, each value verified and redone exactly if it fails (fo_math.h)
             am = fmaxf(am, 1e-12f);
-            if (kQuick) {  // quick forms, each value verified and redone exactly if it fails (fo_math.h)
-                const float av_quick = fmaxf(hw::sqrt(vmax), 1e-12f);
-                av = fmaxf(sqrt_corrected(vmax), 1e-12f);
-                for (int k = 0; k < cnt; ++k) {
-                    ((uint8_t*)mom)[g0 + k] = (uint8_t)quantize_mom_code_verified(m[k], am);
-                    ((uint8_t*)var)[g0 + k] = (uint8_t)quantize_var_code_verified(v[k], av_quick, av);
-                }
-            } else {
-                av = fmaxf(av, 1e-12f);
-                const float ram = hw::rcp(am), rav = hw::rcp(av);
-                for (int k = 0; k < cnt; ++k) {
-                    ((uint8_t*)mom)[g0 + k] = (uint8_t)quantize_mom_code(m[k], am, ram);
-                    ((uint8_t*)var)[g0 + k] = (uint8_t)quantize_var_code(r[k], av, rav);
-                }
+            const float av_quick = fmaxf(hw::sqrt(vmax), 1e-12f);
+            const float av = fmaxf(sqrt_corrected(vmax), 1e-12f);
+            for (int k = 0; k < cnt; ++k) {
+                ((uint8_t*)mom)[g0 + k] = (uint8_t)quantize_mom_code_verified(m[k], am);
+                ((uint8_t*)var)[g0 + k] = (uint8_t)quantize_var_code_verified(v[k], av_quick, av);
             }
             mom_scales[group] = f32_to_f16(am);
             var_scales[group] = f32_to_f16(av);
@@ -192,14 +188,22 @@ template <template <int, int, bool> class F, class... A> int dispatch(int dtype,
 
 template <int DT, int EB, bool Q> struct AdamRun {
     static void run(void* mom, void* ms, void* var, void* vs, void* param, const void* grad, void* ecc, int64_t n,
-                    const AdamHyper& h, int decoupled, int exact) {
-        const bool ex = exact < 0 ? AdamExact<DT, EB>::value : exact != 0;
-        if (decoupled) {
-            if (ex) adam_tensor<DT, EB, Q, true, true>(mom, (uint16_t*)ms, var, (uint16_t*)vs, param, grad, ecc, n, h);
-            else adam_tensor<DT, EB, Q, true, false>(mom, (uint16_t*)ms, var, (uint16_t*)vs, param, grad, ecc, n, h);
+                    const AdamHyper& h, int decoupled, int exact, int64_t* flagged) {
+        // the folded update exists only for the variants that can vouch for it (AdamExact names the others)
+        const bool ex = AdamExact<DT, EB>::value || exact > 0 || !h.folded_ok;
+        uint16_t* ms16 = (uint16_t*)ms;
+        uint16_t* vs16 = (uint16_t*)vs;
+        if constexpr (AdamExact<DT, EB>::value) {
+            if (decoupled) adam_tensor<DT, EB, Q, true, true>(mom, ms16, var, vs16, param, grad, ecc, n, h, flagged);
+            else adam_tensor<DT, EB, Q, false, true>(mom, ms16, var, vs16, param, grad, ecc, n, h, flagged);
         } else {
-            if (ex) adam_tensor<DT, EB, Q, false, true>(mom, (uint16_t*)ms, var, (uint16_t*)vs, param, grad, ecc, n, h);
-            else adam_tensor<DT, EB, Q, false, false>(mom, (uint16_t*)ms, var, (uint16_t*)vs, param, grad, ecc, n, h);
+            if (decoupled) {
+                if (ex) adam_tensor<DT, EB, Q, true, true>(mom, ms16, var, vs16, param, grad, ecc, n, h, flagged);
+                else adam_tensor<DT, EB, Q, true, false>(mom, ms16, var, vs16, param, grad, ecc, n, h, flagged);
+            } else {
+                if (ex) adam_tensor<DT, EB, Q, false, true>(mom, ms16, var, vs16, param, grad, ecc, n, h, flagged);
+                else adam_tensor<DT, EB, Q, false, false>(mom, ms16, var, vs16, param, grad, ecc, n, h, flagged);
+            }
         }
     }
 };
@@ -218,13 +222,36 @@ extern "C" {
 void hm_set_noise(int v) { fo_math_host_noise = v; }
 
 // Arguments as fo_adam_step (include/flashoptim_hip.h) without the stream; host pointers.
-// exact: -1 = the choice the kernels make for this variant, 0 = folded update, 1 = operation by operation.
+// exact: <= 0 = the choice the kernels make for this variant (fo_adam_step), 1 = operation by operation on every
+// element (fo_adam_step_exact).  flagged (may be null): receives the number of elements whose folded update was
+// redone operation by operation.
 int hm_adam_step(void* mom, void* mom_scales, void* var, void* var_scales, void* param, const void* grad, void* ecc,
                  int64_t n, int dtype, int ecc_bytes, int quantized, float lr, float beta1, float beta2, float eps,
-                 float weight_decay, int decoupled, int step, int exact) {
+                 float weight_decay, int decoupled, int step, int exact, int64_t* flagged) {
     const AdamHyper h = make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step);
-    return dispatch<AdamRun>(dtype, ecc_bytes, quantized, mom, mom_scales, var, var_scales, param, grad, ecc, n, h, decoupled, exact);
+    if (flagged) *flagged = 0;
+    return dispatch<AdamRun>(dtype, ecc_bytes, quantized, mom, mom_scales, var, var_scales, param, grad, ecc, n, h, decoupled, exact, flagged);
 }
+// The folded update of bf16 parameters with a 1-byte ECC and quantised states WITHOUT the repair: the fp32 results
+// and which elements the guard flags.  Changes nothing in place.
+void hm_adam_folded_update(const void* mom, const void* mom_scales, const void* var, const void* var_scales, const void* param,
+                           const void* grad, const void* ecc, int64_t n, float lr, float beta1, float beta2, float eps,
+                           float weight_decay, int decoupled, int step, float* p_out, uint8_t* redo_out) {
+    const AdamHyper h = make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step);
+    for (int64_t i = 0; i < n; ++i) {
+        const float sm = f16_to_f32(((const uint16_t*)mom_scales)[i >> 5]), sv = f16_to_f32(((const uint16_t*)var_scales)[i >> 5]);
+        const float p0 = read_master<DT_BF16, 1>(param, ecc, i);
+        float gr = load_elem<DT_BF16>(grad, i);
+        if (!decoupled) gr = gr + p0 * h.wd;
+        float mn, vn;
+        adam_moments_quantized(gr, kTable.v[((const uint8_t*)mom)[i]], sm, (float)((const uint8_t*)var)[i], sv, h, mn, vn);
+        bool redo;
+        p_out[i] = decoupled ? adam_apply_folded<true>(p0, mn, hw::sqrt(vn), h, AdamFoldedGuard<DT_BF16, 1>::value, redo)
+                             : adam_apply_folded<false>(p0, mn, hw::sqrt(vn), h, AdamFoldedGuard<DT_BF16, 1>::value, redo);
+        redo_out[i] = redo ? 1 : 0;
+    }
+}
+void hm_code_over_255(float* out) { for (int q = 0; q < 256; ++q) out[q] = code_over_255((float)q); }
 
 // Arguments as fo_momentum_step without the stream.
 int hm_momentum_step(void* mom, void* mom_scales, void* param, const void* grad, void* ecc, int64_t n, int dtype,

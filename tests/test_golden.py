@@ -144,20 +144,18 @@ def test_hip_ecc_matches_vectors(name):
     assert _same(k.reconstruct_fp32_param(narrow, ecc).cpu(), _get(f"{name}/joined"))
 
 
-def _check_step(name, quantized, got, want, info, state_names, exact):
-    """exact: every output bit equals the committed vector (all kernels but Adam on bf16 / fp16 parameters)."""
+def _check_step(name, got, want, state_names, exact):
+    """Moments, codes and scales: every bit equals the committed vector.  exact: parameters and ECC too (every kernel
+    but Adam with the guarded folded update, whose master weights stay within one unit of master precision)."""
+    for key in tuple(k for pair in state_names for k in pair):
+        if want.get(key) is not None:
+            assert parity.bits_equal(got[key], want[key]), f"{name} {key}: bits differ"
     if exact:
-        for key in ("p", "ecc") + tuple(k for pair in state_names for k in pair):
+        for key in ("p", "ecc"):
             if want.get(key) is not None:
                 assert parity.bits_equal(got[key], want[key]), f"{name} {key}: bits differ"
         return
-    parity.check_master(got["p"], got["ecc"], want["p"], want["ecc"], name, step_size=info["update_scale"])
-    for key, skey in state_names:
-        if quantized:
-            parity.check_codes(got[key], want[key], f"{name} {key}")
-            parity.check_scales(got[skey], want[skey], f"{name} {skey}")
-        else:
-            assert parity.bits_equal(got[key], want[key]), f"{name} {key}: unquantised state differs"
+    parity.check_master(got["p"], got["ecc"], want["p"], want["ecc"], name)
 
 
 @pytest.mark.gpu
@@ -168,14 +166,11 @@ def test_hip_adam_step_matches_vectors(name, dt, ec, quantized, decoupled):
     want = _expected(name, dt, quantized, ("p", "ecc", "m", "ms", "v", "vs"))
     hp = G.ADAM_HP
     wd = 0.01 * hp["lr"] if decoupled else 0.01
-    b = _adam_inputs(name, dt, quantized)   # the oracle's intermediates give the size of the update
-    mom = T.MomentState(b["m"], b["ms"]) if quantized else T.MomentState(plain=b["m"])
-    var = T.MomentState(b["v"], b["vs"]) if quantized else T.MomentState(plain=b["v"])
-    info = T.adam_step_ref(mom, var, b["p"], b["g"], b["ecc"], hp["lr"], hp["beta1"], hp["beta2"], hp["eps"], wd, decoupled, 3)
     a = {key: _dev(t) for key, t in _adam_inputs(name, dt, quantized).items()}
     k._fused_adam_step(a["m"], a["ms"], a["v"], a["vs"], a["p"], a["g"], a["ecc"], hp["lr"], hp["beta1"], hp["beta2"], hp["eps"],
                        wd, decoupled, 3, quantize_optim_states=quantized)
-    _check_step(name, quantized, a, want, info, (("m", "ms"), ("v", "vs")), exact=dt == torch.float32)
+    folded = dt != "f32" and (ec == "none" or (dt == "bf16" and ec == "i8"))  # the guarded folded update
+    _check_step(name, a, want, (("m", "ms"), ("v", "vs")), exact=not folded)
 
 
 @pytest.mark.gpu
@@ -184,9 +179,6 @@ def test_hip_momentum_step_matches_vectors(name, dt, ec, quantized, kw):
     from flashoptim_amd import kernels as k
 
     want = _expected(name, dt, quantized, ("p", "ecc", "m", "ms"))
-    b = _mom_inputs(name, dt, quantized)
-    mom = T.MomentState(b["m"], b["ms"]) if quantized else T.MomentState(plain=b["m"])
-    info = T.momentum_step_ref(mom, b["p"], b["g"], b["ecc"], **kw)
     a = {key: _dev(t) for key, t in _mom_inputs(name, dt, quantized).items()}
     k._fused_momentum_step(a["m"], a["ms"], a["p"], a["g"], a["ecc"], quantize_optim_states=quantized, **kw)
-    _check_step(name, quantized, a, want, info, (("m", "ms"),), exact=True)
+    _check_step(name, a, want, (("m", "ms"),), exact=True)

@@ -78,18 +78,18 @@ def _oracle_check(kind, before, after, step, what):
     p, g, ecc = before.p.cpu(), before.g.cpu(), before.ecc.cpu()
     states = [T.MomentState(c.cpu(), s.cpu()) for c, s in zip(before.codes, before.scales)]
     if kind == "adam":
-        info = T.adam_step_ref(states[0], states[1], p, g, ecc, ADAM["lr"], ADAM["beta1"], ADAM["beta2"], ADAM["eps"],
-                               ADAM["weight_decay"], ADAM["decoupled"], step)
+        T.adam_step_ref(states[0], states[1], p, g, ecc, ADAM["lr"], ADAM["beta1"], ADAM["beta2"], ADAM["eps"],
+                        ADAM["weight_decay"], ADAM["decoupled"], step)
     else:
-        info = T.momentum_step_ref(states[0], p, g, ecc, **LION)
+        T.momentum_step_ref(states[0], p, g, ecc, **LION)
+    # codes and scales equal the oracle's bit for bit under every kernel
+    for i, st in enumerate(states):
+        assert parity.bits_equal(after.codes[i], st.codes) and parity.bits_equal(after.scales[i], st.scales), f"{what} state{i}"
     if kind != "adam":  # the momentum kernels equal the oracle bit for bit
         assert parity.bits_equal(after.p, p) and parity.bits_equal(after.ecc, ecc), f"{what}: parameter or ECC bits differ"
-        assert parity.bits_equal(after.codes[0], states[0].codes) and parity.bits_equal(after.scales[0], states[0].scales), what
         return
-    parity.check_master(after.p, after.ecc, p, ecc, what, step_size=info["update_scale"])
-    for i in range(2):
-        parity.check_codes(after.codes[i], states[i].codes, f"{what} state{i}")
-        parity.check_scales(after.scales[i], states[i].scales, f"{what} state{i}")
+    # Adam on bf16 parameters with a 1-byte ECC: guarded folded update, master weights within one unit
+    parity.check_master(after.p, after.ecc, p, ecc, what)
 
 
 def _run(kind, n, n_windows, extra=()):
