@@ -48,8 +48,7 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
 
     float p[EPL], m[EPL], r[EPL], v[EPL];
     read_master<DT, ECCB, EPL>(p, raw.p, raw.e, lut);
-    bool redo[EPL];
-    bool any_redo = false;
+    float slack[EPL];  // folded update: negative where the element has to be redone operation by operation
 
 #pragma unroll
     for (int k = 0; k < EPL; ++k) {
@@ -69,22 +68,25 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
         } else {
             // folded update; `redo` marks the elements it cannot vouch for (fo_math.h).  The old weight stays in
             // raw.p / raw.e for the repair below.
-            p[k] = adam_apply_folded<DECOUPLED>(p[k], mn, rk, h, AdamFoldedGuard<DT, ECCB>::value, redo[k]);
-            any_redo |= redo[k];
+            p[k] = adam_apply_folded<DECOUPLED>(p[k], mn, rk, h, AdamFoldedGuard<DT, ECCB>::value, slack[k]);
         }
         m[k] = mn; r[k] = rk; v[k] = vn;
     }
     if constexpr (!EXACT) {
         // The flagged elements again, operation by operation.  A wavefront with no flagged element branches past
         // this; otherwise only the element positions that are flagged in some lane are redone.
-        if (__builtin_amdgcn_ballot_w64(any_redo) != 0) {
+        float least = slack[0];
+#pragma unroll
+        for (int k = 1; k < EPL; ++k) least = fminf(least, slack[k]);
+        if (__builtin_amdgcn_ballot_w64(adam_folded_is_flagged(least)) != 0) {
 #pragma unroll
             for (int k = 0; k < EPL; ++k) {
-                if (__builtin_amdgcn_ballot_w64(redo[k]) != 0) {
+                const bool redo = adam_folded_is_flagged(slack[k]);
+                if (__builtin_amdgcn_ballot_w64(redo) != 0) {
                     float pk = master_of<DT, ECCB, EPL>(raw.p, raw.e, k, lut);
                     if constexpr (DECOUPLED) pk = pk * h.one_m_wd;
                     const float pe = adam_apply_exact(pk, m[k], v[k], h);
-                    if (redo[k]) p[k] = pe;
+                    if (redo) p[k] = pe;
                 }
             }
         }
@@ -131,7 +133,7 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
 // by default; the *_exact entry points ask for it on every variant).
 template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT = AdamExact<DT, ECCB>::value> struct AdamOp {
     using Hyper = AdamHyper;
-    static constexpr int kLutTables = ECCB == 1 ? 2 : (QUANT ? 1 : 0);  // LDS code tables (fo_device.h)
+    static constexpr int kLutMask = (QUANT ? 1 << kTableMom : 0) | (ECCB == 1 ? 1 << kTableEcc : 0);  // LDS code tables
     static constexpr int kDtype = DT;
     // measured on MI355X with the 8B-parameter step and this file's ILP-oriented instruction schedule, over the
     // residencies the LDS units allow (fo_step.h): 16 for 2-byte parameters (3.6-4.6 KiB of loads per wavefront; 14
@@ -143,8 +145,20 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT = AdamExact<D
     // a cap of five is as erratic, so that variant stays uncapped, like fp32 (a cap costs a point there).  The
     // operation-by-operation update on 2-byte parameters gains two points from its cap of five on every box.
     static constexpr bool kNarrowExact = EXACT && DT != DT_F32;
-    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 18 : (kNarrowExact ? 20 : 16);
-    static constexpr int kMaxWavesPerSimd = DT == DT_F32 ? 8 : (kNarrowExact ? 5 : (ECCB == 2 ? 8 : 4));
+#ifndef FO_EXACT_WG
+#define FO_EXACT_WG 20
+#endif
+#ifndef FO_EXACT_WAVES
+#define FO_EXACT_WAVES 5
+#endif
+#ifndef FO_FOLDED_WG
+#define FO_FOLDED_WG 16
+#endif
+#ifndef FO_FOLDED_WAVES
+#define FO_FOLDED_WAVES 4
+#endif
+    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 18 : (kNarrowExact ? FO_EXACT_WG : FO_FOLDED_WG);
+    static constexpr int kMaxWavesPerSimd = DT == DT_F32 ? 8 : (kNarrowExact ? FO_EXACT_WAVES : FO_FOLDED_WAVES);
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {
@@ -166,7 +180,7 @@ struct StreamsHyper { uint32_t mask; };
 
 template <int DT, int ECCB, bool QUANT> struct AdamStreamsOp {
     using Hyper = StreamsHyper;
-    static constexpr int kLutTables = 0;
+    static constexpr int kLutMask = 0;
     static constexpr int kDtype = DT;
     // where this copy streams fastest on MI355X with the 8B-parameter list: 16 with 1-byte ECC (14 and 18 are three
     // to four points slower), 14 with 2-byte ECC (16 one point slower); fp32 parameters (256 elements and 2.5 KiB per

@@ -311,38 +311,45 @@ __device__ __forceinline__ void convert_pack8(const float (&a)[4], const float (
 // 8-bit group codec pieces used by the fused kernels
 // ------------------------------------------------------------------------------------------------
 
-template <int CTRL> __device__ __forceinline__ float dpp_move(float x) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
-}
+// max(x, x of the lane that the DPP control selects) in one instruction.  (Written as a DPP move followed by fmaxf
+// the compiler emits the move, one or two canonicalising maxes and the max itself.)  v_max_f32 returns the other
+// operand when one is a NaN, as fmaxf does.  A DPP source register written by the preceding VALU instruction
+// needs two wait states, and the hazard recogniser does not look inside asm: hence the s_nop.
+#define FO_DPP_MAX(CTRL)                                                                                           \
+    asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1" : "=&v"(r) : "v"(x))
 
 // max over the 32/EPL neighbouring lanes that share one quantisation group; every lane gets the result
 template <int EPL> __device__ __forceinline__ float group_max(float x) {
-    x = fmaxf(x, dpp_move<0xB1>(x));  // quad_perm [1,0,3,2]
-    x = fmaxf(x, dpp_move<0x4E>(x));  // quad_perm [2,3,0,1]: now the max of each aligned group of 4 lanes
-    if constexpr (EPL == 4) x = fmaxf(x, dpp_move<0x141>(x));  // row_half_mirror: swaps the two quads of each 8 lanes
+    float r;
+    FO_DPP_MAX("quad_perm:[1,0,3,2]"); x = r;
+    FO_DPP_MAX("quad_perm:[2,3,0,1]"); x = r;  // now the max of each aligned group of 4 lanes
+    if constexpr (EPL == 4) { FO_DPP_MAX("row_half_mirror"); x = r; }  // swaps the two quads of each 8 lanes
     return x;
 }
+#undef FO_DPP_MAX
 
 // The code tables (fo_math.h) in device memory, one instance per parameter dtype.
 template <int DT> __device__ const StepTables<DT> kStepTables = StepTables<DT>();
 
-// The tables live in LDS during a kernel (1 KiB each, no replication: a few conflicted reads cost less than
-// filling a bank-replicated copy, because every short-lived workgroup fills its own).  A workgroup is one
-// wavefront; it fills each table with one 128-bit load per lane that writes straight into LDS (lane l delivers
-// entries 4l .. 4l+3; no registers, no ds_write).  The loads are issued before the workgroup's streaming loads and
-// the first lookup only waits for them, not for the streams issued after them.
-// TABLES: 1 = first-moment codes, 2 = also the int8 ECC fractions.
-template <int TABLES> struct StepLut {
-    static constexpr int kFloats = TABLES > 0 ? 256 * TABLES : 4;
+// The tables a kernel uses live in LDS while it runs (1 KiB each at fixed places, no replication: a few conflicted
+// reads cost less than filling a bank-replicated copy, because every short-lived workgroup fills its own).  A
+// workgroup is one wavefront; it fills each table with one 128-bit load per lane that writes straight into LDS
+// (lane l delivers entries 4l .. 4l+3; no registers, no ds_write).  The loads are issued before the workgroup's
+// streaming loads and the first lookup only waits for them, not for the streams issued after them.
+// MASK: bit t set = table t (kTableMom, kTableEcc) is used.
+template <int MASK> struct StepLut {
+    static constexpr int kTables = (MASK & 2) ? 2 : (MASK & 1);  // LDS reaches up to the last one used
+    static constexpr int kFloats = kTables > 0 ? 256 * kTables : 4;
     __device__ __forceinline__ static void fill(float* lut, const float* table) {
 #pragma unroll
-        for (int t = 0; t < TABLES; ++t)
-            __builtin_amdgcn_global_load_lds((const FO_GLOBAL void*)(table + 256 * t + (threadIdx.x & 63) * 4),
-                                             (__attribute__((address_space(3))) void*)(lut + 256 * t), 16, 0, 0);
+        for (int t = 0; t < kTableCount; ++t)
+            if ((MASK >> t) & 1)
+                __builtin_amdgcn_global_load_lds((const FO_GLOBAL void*)(table + 256 * t + (threadIdx.x & 63) * 4),
+                                                 (__attribute__((address_space(3))) void*)(lut + 256 * t), 16, 0, 0);
     }
 };
-__device__ __forceinline__ float lookup_mom(const float* lut, u32 byte) { return lut[byte]; }
-__device__ __forceinline__ float lookup_ecc(const float* lut, u32 byte) { return lut[256 + byte]; }
+__device__ __forceinline__ float lookup_mom(const float* lut, u32 byte) { return lut[256 * kTableMom + byte]; }
+__device__ __forceinline__ float lookup_ecc(const float* lut, u32 byte) { return lut[256 * kTableEcc + byte]; }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }  // RTNE

@@ -195,20 +195,24 @@ template <int DT, int ECCB, bool CLAMP> FO_FN u32 ecc_split_bits(float p, float 
 // 8-bit group codec
 // ------------------------------------------------------------------------------------------------
 
-// The two code tables of the step kernels, evaluated by the compiler (IEEE, round to nearest):
-//   v[b]        first-moment value of signed code byte b before the group scale, (q/127) / (2 - |q/127|) with
+// The two code tables of the step kernels, evaluated by the compiler (IEEE, round to nearest), 256 entries each,
+// indexed by the code byte:
+//   kTableMom   first-moment value of signed code byte b before the group scale, (q/127) / (2 - |q/127|) with
 //               each operation correctly rounded (ref:2332-2336);
-//   v[256 + b]  (q/127) * 2^-(mant+1) for an int8 ECC byte b, the division correctly rounded (ref:2772): the
+//   kTableEcc   (q/127) * 2^-(mant+1) for an int8 ECC byte b, the division correctly rounded (ref:2772): the
 //               factor that multiplies 2^E in ecc_join_fraction.  The scaling by a power of two is exact.
+// (The second-moment value q / 255 is formed arithmetically, code_over_255: a third table saved two instructions
+// per element and cost a lookup, with no gain in step time.)
+enum { kTableMom = 0, kTableEcc = 1, kTableCount = 2 };
 template <int DT> struct StepTables {
-    float v[512];
+    float v[256 * kTableCount];
     constexpr StepTables() : v() {
         for (int b = 0; b < 256; ++b) {
             const int q = b < 128 ? b : b - 256;
             const float y = (float)q / 127.0f;
             const float a = y < 0.0f ? -y : y;
-            v[b] = y / (2.0f - a);
-            v[256 + b] = y * (1.0f / (float)(1 << (DTypeInfo<DT>::mant + 1)));
+            v[256 * kTableMom + b] = y / (2.0f - a);
+            v[256 * kTableEcc + b] = y * (1.0f / (float)(1 << (DTypeInfo<DT>::mant + 1)));
         }
     }
 };
@@ -262,8 +266,12 @@ FO_FN float quantize_mom_quick(float m, float am) {
     return hw::fma(t, 254.0f, 0.5f + kQuickMarginMom);
 }
 FO_FN float quantize_var_quick(float r, float rav255) { return hw::fma(r, rav255, 0.5f + kQuickMarginVar); }
-// floor(x) is the exact form's code unless x (a quick value, margin included) lies within the margin of an integer.
-FO_FN bool quick_value_is_safe(float x, float margin) { return hw::fract(x) >= 2.0f * margin; }
+// floor(x) is the exact form's code unless x (a quick value, margin included) lies within the margin of an integer:
+// the value is safe when fract(x) >= 2 margin.  quick_value_slack is that fractional part; callers that hold several
+// values compare the smallest slack once and look at the single values only when that fails.
+FO_FN float quick_value_slack(float x) { return hw::fract(x); }
+FO_FN bool quick_slack_is_safe(float slack, float margin) { return slack >= 2.0f * margin; }
+FO_FN bool quick_value_is_safe(float x, float margin) { return quick_slack_is_safe(quick_value_slack(x), margin); }
 // One value through quick form, test and, if need be, exact form (what the kernels do, element by element).
 //   av_quick / av_exact: hw::sqrt and sqrt_corrected of the group's largest v; v: the element's second moment.
 FO_FN u32 quantize_mom_code_verified(float m, float am) {
@@ -388,14 +396,17 @@ template <int DT, int ECCB> struct AdamFoldedGuard {
     static_assert(!AdamExact<DT, ECCB>::value, "the folded update is not offered for this variant");
     static constexpr float value = ECCB == 1 ? 16.0f : (DT == DT_BF16 ? 4096.0f : 512.0f);
 };
+// Returns the new weight; `slack` receives guard * |p_new| - |update|, negative for a flagged element (callers that
+// hold several elements take the smallest slack, test it once and look at the single ones only when that fails).
 template <bool DECOUPLED>
-FO_FN float adam_apply_folded(float p, float mn, float r, const AdamHyper& h, float guard, bool& redo) {
+FO_FN float adam_apply_folded(float p, float mn, float r, const AdamHyper& h, float guard, float& slack) {
     const float neg_den = hw::fma(r, h.neg_den_scale, h.neg_den_bias);
     const float u = mn * hw::rcp(neg_den);
     const float pn = DECOUPLED ? hw::fma(p, h.one_m_wd, u) : p + u;
-    redo = fabsf(pn) * guard < fabsf(u);
+    slack = hw::fma(fabsf(pn), guard, -fabsf(u));
     return pn;
 }
+FO_FN bool adam_folded_is_flagged(float slack) { return slack < 0.0f; }
 
 // ------------------------------------------------------------------------------------------------
 // SGD / SGDW / Nesterov / Lion element update (ref:1624-1683, 1447-1465)

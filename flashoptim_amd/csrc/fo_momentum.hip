@@ -85,7 +85,7 @@ __device__ __forceinline__ void momentum_finish(const TensorPtrs& t, Where w, Mo
 
 template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumOp {
     using Hyper = MomentumHyper;
-    static constexpr int kLutTables = ECCB == 1 ? 2 : ((QUANT && KIND != KIND_PLAIN) ? 1 : 0);  // LDS code tables (fo_device.h)
+    static constexpr int kLutMask = ((QUANT && KIND != KIND_PLAIN) ? 1 << kTableMom : 0) | (ECCB == 1 ? 1 << kTableEcc : 0);  // LDS code tables
     static constexpr int kDtype = DT;
     // measured on MI355X (3 KiB of loads per wavefront) over the residencies the LDS units allow (fo_step.h: 18, 21,
     // 25, 32 around here): the 8B list is as fast at 21 as at 25, 4096 ragged tensors need 25 or more; capping the
@@ -113,7 +113,7 @@ struct MomentumStreamsHyper { uint32_t mask; };
 
 template <int DT, int ECCB, bool QUANT> struct MomentumStreamsOp {
     using Hyper = MomentumStreamsHyper;
-    static constexpr int kLutTables = 0;
+    static constexpr int kLutMask = 0;
     static constexpr int kDtype = DT;
     // measured on MI355X: the 8B-parameter list streams fastest at 14 (83.2 %; 16: 82.0 %, 18: 79.6 %), 4096 ragged
     // tensors at 16 (81.8 %; 14: 80.2 %, 18: 81.5 %)

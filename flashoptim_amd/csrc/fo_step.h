@@ -8,7 +8,7 @@
 // that each touch every stream once than with larger or persistent ones.  The multi-tensor grid addresses work
 // through a chunk table in units of 4096-element tiles; a tile is an integer number of spans.  A quantisation
 // group is 32/EPL neighbouring lanes, so the group absmax is in-register maxes plus two or three DPP moves.
-// LDS only holds the two 256-entry code tables (first-moment code -> value, int8 ECC code -> fraction).
+// LDS only holds the 256-entry code tables (moment code -> value, int8 ECC code -> fraction).
 //
 // "ref:" cites /root/reference/flashoptim/optimizers.py.
 #pragma once
@@ -104,24 +104,25 @@ template <int EPL> __device__ __forceinline__ void set_code(Pack<1, EPL>& out, i
 template <int EPL>
 __device__ __forceinline__ void quantize_mom_quick_verified(const float (&m)[EPL], float am, Pack<1, EPL>& out) {
     static_assert(EPL == 8, "two dwords of codes per lane");
-    float x[8];
-    bool redo[8];
-    bool any = false;
+    float x[8], slack[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
         x[k] = quantize_mom_quick(m[k], am);
-        redo[k] = !quick_value_is_safe(x[k], kQuickMarginMom);
-        any |= redo[k];
+        slack[k] = quick_value_slack(x[k]);
     }
+    float least = slack[0];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) least = fminf(least, slack[k]);
     const float lo[4] = {x[0], x[1], x[2], x[3]}, hi[4] = {x[4], x[5], x[6], x[7]};
     convert_pack8<kFloor, kFloor>(lo, hi, out.w[0], out.w[1]);
-    if (__builtin_amdgcn_ballot_w64(any) != 0) {
+    if (__builtin_amdgcn_ballot_w64(!quick_slack_is_safe(least, kQuickMarginMom)) != 0) {
         const float ram = hw::rcp(am);
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            if (__builtin_amdgcn_ballot_w64(redo[k]) != 0) {
+            const bool redo = !quick_slack_is_safe(slack[k], kQuickMarginMom);
+            if (__builtin_amdgcn_ballot_w64(redo) != 0) {
                 const u32 code = quantize_mom_code(m[k], am, ram);
-                if (redo[k]) set_code<EPL>(out, k, code);
+                if (redo) set_code<EPL>(out, k, code);
             }
         }
     }
@@ -132,24 +133,25 @@ __device__ __forceinline__ void quantize_var_quick_verified(const float (&v)[EPL
                                                             float av_exact, Pack<1, EPL>& out) {
     static_assert(EPL == 8, "two dwords of codes per lane");
     const float rav255 = hw::rcp(av_quick) * 255.0f;
-    float x[8];
-    bool redo[8];
-    bool any = false;
+    float x[8], slack[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
         x[k] = quantize_var_quick(r[k], rav255);
-        redo[k] = !quick_value_is_safe(x[k], kQuickMarginVar);
-        any |= redo[k];
+        slack[k] = quick_value_slack(x[k]);
     }
+    float least = slack[0];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) least = fminf(least, slack[k]);
     const float lo[4] = {x[0], x[1], x[2], x[3]}, hi[4] = {x[4], x[5], x[6], x[7]};
     convert_pack8<kTrunc, kTrunc>(lo, hi, out.w[0], out.w[1]);
-    if (__builtin_amdgcn_ballot_w64(any) != 0) {
+    if (__builtin_amdgcn_ballot_w64(!quick_slack_is_safe(least, kQuickMarginVar)) != 0) {
         const float rav = hw::rcp(av_exact);
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            if (__builtin_amdgcn_ballot_w64(redo[k]) != 0) {
+            const bool redo = !quick_slack_is_safe(slack[k], kQuickMarginVar);
+            if (__builtin_amdgcn_ballot_w64(redo) != 0) {
                 const u32 code = quantize_var_code(sqrt_corrected(v[k]), av_exact, rav);
-                if (redo[k]) set_code<EPL>(out, k, code);
+                if (redo) set_code<EPL>(out, k, code);
             }
         }
     }
@@ -160,29 +162,31 @@ __device__ __forceinline__ void quantize_mom_var_quick_verified(const float (&m)
                                                                 const float (&r)[4], float av_quick, float av_exact,
                                                                 Pack<1, 4>& mout, Pack<1, 4>& vout) {
     const float rav255 = hw::rcp(av_quick) * 255.0f;
-    float xm[4], xv[4];
-    bool redo_m[4], redo_v[4];
-    bool any = false;
+    float xm[4], xv[4], slack_m[4], slack_v[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         xm[k] = quantize_mom_quick(m[k], am);
         xv[k] = quantize_var_quick(r[k], rav255);
-        redo_m[k] = !quick_value_is_safe(xm[k], kQuickMarginMom);
-        redo_v[k] = !quick_value_is_safe(xv[k], kQuickMarginVar);
-        any |= redo_m[k] | redo_v[k];
+        slack_m[k] = quick_value_slack(xm[k]);
+        slack_v[k] = quick_value_slack(xv[k]);
     }
+    const float least_m = fminf(fminf(slack_m[0], slack_m[1]), fminf(slack_m[2], slack_m[3]));
+    const float least_v = fminf(fminf(slack_v[0], slack_v[1]), fminf(slack_v[2], slack_v[3]));
     convert_pack8<kFloor, kTrunc>(xm, xv, mout.w[0], vout.w[0]);
+    const bool any = !quick_slack_is_safe(least_m, kQuickMarginMom) | !quick_slack_is_safe(least_v, kQuickMarginVar);
     if (__builtin_amdgcn_ballot_w64(any) != 0) {
         const float ram = hw::rcp(am), rav = hw::rcp(av_exact);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            if (__builtin_amdgcn_ballot_w64(redo_m[k]) != 0) {
+            const bool redo_m = !quick_slack_is_safe(slack_m[k], kQuickMarginMom);
+            const bool redo_v = !quick_slack_is_safe(slack_v[k], kQuickMarginVar);
+            if (__builtin_amdgcn_ballot_w64(redo_m) != 0) {
                 const u32 code = quantize_mom_code(m[k], am, ram);
-                if (redo_m[k]) set_code<4>(mout, k, code);
+                if (redo_m) set_code<4>(mout, k, code);
             }
-            if (__builtin_amdgcn_ballot_w64(redo_v[k]) != 0) {
+            if (__builtin_amdgcn_ballot_w64(redo_v) != 0) {
                 const u32 code = quantize_var_code(sqrt_corrected(v[k]), av_exact, rav);
-                if (redo_v[k]) set_code<4>(vout, k, code);
+                if (redo_v) set_code<4>(vout, k, code);
             }
         }
     }
@@ -250,9 +254,9 @@ __device__ __forceinline__ void run_span(const TensorPtrs& t, int64_t base, bool
 #define FO_WAVES_ATTR __attribute__((amdgpu_waves_per_eu(1, Op::kMaxWavesPerSimd)))
 template <class Op>
 __global__ __launch_bounds__(kBlockThreads) FO_WAVES_ATTR void step_single_kernel(TensorPtrs t, typename Op::Hyper h) {
-    __shared__ __align__(16) float lut[StepLut<Op::kLutTables>::kFloats];
+    __shared__ __align__(16) float lut[StepLut<Op::kLutMask>::kFloats];
     const int64_t base = (int64_t)blockIdx.x * Span<Op>::kElems;
-    if constexpr (Op::kLutTables > 0) StepLut<Op::kLutTables>::fill(lut, kStepTables<Op::kDtype>.v);
+    if constexpr (Op::kLutMask != 0) StepLut<Op::kLutMask>::fill(lut, kStepTables<Op::kDtype>.v);
     run_span<Op>(t, base, all_aligned16(t), h, lut);
 }
 
@@ -260,12 +264,12 @@ __global__ __launch_bounds__(kBlockThreads) FO_WAVES_ATTR void step_single_kerne
 template <class Op>
 __global__ __launch_bounds__(kBlockThreads) FO_WAVES_ATTR void step_multi_kernel(const fo_tensor_desc* __restrict__ descs,
                                                                    const fo_chunk* __restrict__ chunks, typename Op::Hyper h) {
-    __shared__ __align__(16) float lut[StepLut<Op::kLutTables>::kFloats];
+    __shared__ __align__(16) float lut[StepLut<Op::kLutMask>::kFloats];
     constexpr int kPerTile = Span<Op>::kPerTile;
     const unsigned b = blockIdx.x;
     const fo_chunk ck = chunks[b / kPerTile];
     const TensorPtrs t = load_desc(descs + ck.tensor);
-    if constexpr (Op::kLutTables > 0) StepLut<Op::kLutTables>::fill(lut, kStepTables<Op::kDtype>.v);
+    if constexpr (Op::kLutMask != 0) StepLut<Op::kLutMask>::fill(lut, kStepTables<Op::kDtype>.v);
     const bool aligned = all_aligned16(t);
     const int64_t in_tile = (int64_t)(b % kPerTile) * Span<Op>::kElems;
     for (int i = 0; i < ck.n_tiles; ++i) {
@@ -385,7 +389,7 @@ template <class Op, class Kernel> const Residency& residency_of(Kernel kernel) {
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
     std::call_once(once[dev], [&] {
         const int forced = debug_workgroups_per_cu();
-        constexpr int kStatic = fo::StepLut<Op::kLutTables>::kFloats * 4;
+        constexpr int kStatic = fo::StepLut<Op::kLutMask>::kFloats * 4;
         cache[dev] = plan_residency(kernel, forced > 0 ? forced : Op::kWorkgroupsPerCu, kStatic, Op::kMaxWavesPerSimd);
     });
     return cache[dev];

@@ -72,7 +72,7 @@ template <int DT> constexpr StepTables<DT> kTables = StepTables<DT>();
 // as read_master in fo_step.h: int8 codes through the fraction table, int16 codes arithmetically
 template <int DT, int ECCB> float read_master(const void* param, const void* ecc, int64_t i) {
     const float w = load_elem<DT>(param, i);
-    if constexpr (ECCB == 1) return ecc_join_fraction<DT>(w, kTables<DT>.v[256 + ((const uint8_t*)ecc)[i]]);
+    if constexpr (ECCB == 1) return ecc_join_fraction<DT>(w, kTables<DT>.v[256 * kTableEcc + ((const uint8_t*)ecc)[i]]);
     if constexpr (ECCB == 2) return ecc_join<DT, ECCB>(w, load_ecc<ECCB>(ecc, i));
     return w;
 }
@@ -100,7 +100,7 @@ void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scale
             if (!DECOUPLED) gr = gr + p0 * h.wd;
             float mn, vn;
             if (QUANT) {
-                adam_moments_quantized(gr, kTable.v[((const uint8_t*)mom)[i]], sm, (float)((const uint8_t*)var)[i], sv, h, mn, vn);
+                adam_moments_quantized(gr, kTable.v[256 * kTableMom + ((const uint8_t*)mom)[i]], sm, (float)((const uint8_t*)var)[i], sv, h, mn, vn);
             } else {
                 adam_moments_plain(gr, load_elem<DT>(mom, i), load_elem<DT>(var, i), h, mn, vn);
             }
@@ -108,9 +108,9 @@ void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scale
             if constexpr (EXACT) {
                 p = adam_apply_exact(DECOUPLED ? p0 * h.one_m_wd : p0, mn, vn, h);
             } else {
-                bool redo;
-                p = adam_apply_folded<DECOUPLED>(p0, mn, hw::sqrt(vn), h, AdamFoldedGuard<DT, ECCB>::value, redo);
-                if (redo) {
+                float slack;
+                p = adam_apply_folded<DECOUPLED>(p0, mn, hw::sqrt(vn), h, AdamFoldedGuard<DT, ECCB>::value, slack);
+                if (adam_folded_is_flagged(slack)) {
                     p = adam_apply_exact(DECOUPLED ? p0 * h.one_m_wd : p0, mn, vn, h);
                     if (flagged) ++*flagged;
                 }
@@ -155,7 +155,7 @@ void momentum_tensor(void* mom, uint16_t* mom_scales, void* param, const void* g
             float p = read_master<DT, ECCB>(param, ecc, i);
             const float gr = load_elem<DT>(grad, i);
             float mo = 0.0f;
-            if (KIND != KIND_PLAIN) mo = QUANT ? kTable.v[((const uint8_t*)mom)[i]] * sm : load_elem<DT>(mom, i);
+            if (KIND != KIND_PLAIN) mo = QUANT ? kTable.v[256 * kTableMom + ((const uint8_t*)mom)[i]] * sm : load_elem<DT>(mom, i);
             momentum_element<KIND>(gr, p, mo, h, m[k]);
             write_master<DT, ECCB>(param, ecc, i, p);
             am = fmaxf(am, fabsf(m[k]));
@@ -244,11 +244,11 @@ void hm_adam_folded_update(const void* mom, const void* mom_scales, const void* 
         float gr = load_elem<DT_BF16>(grad, i);
         if (!decoupled) gr = gr + p0 * h.wd;
         float mn, vn;
-        adam_moments_quantized(gr, kTable.v[((const uint8_t*)mom)[i]], sm, (float)((const uint8_t*)var)[i], sv, h, mn, vn);
-        bool redo;
-        p_out[i] = decoupled ? adam_apply_folded<true>(p0, mn, hw::sqrt(vn), h, AdamFoldedGuard<DT_BF16, 1>::value, redo)
-                             : adam_apply_folded<false>(p0, mn, hw::sqrt(vn), h, AdamFoldedGuard<DT_BF16, 1>::value, redo);
-        redo_out[i] = redo ? 1 : 0;
+        adam_moments_quantized(gr, kTable.v[256 * kTableMom + ((const uint8_t*)mom)[i]], sm, (float)((const uint8_t*)var)[i], sv, h, mn, vn);
+        float slack;
+        p_out[i] = decoupled ? adam_apply_folded<true>(p0, mn, hw::sqrt(vn), h, AdamFoldedGuard<DT_BF16, 1>::value, slack)
+                             : adam_apply_folded<false>(p0, mn, hw::sqrt(vn), h, AdamFoldedGuard<DT_BF16, 1>::value, slack);
+        redo_out[i] = adam_folded_is_flagged(slack) ? 1 : 0;
     }
 }
 void hm_code_over_255(float* out) { for (int q = 0; q < 256; ++q) out[q] = code_over_255((float)q); }
@@ -285,8 +285,8 @@ void hm_quantize_group(const float* m, const float* r, uint8_t* qm, uint8_t* qv,
 void hm_ecc_fraction_table(int dtype, float* table_out, float* arithmetic_out) {
     for (int b = 0; b < 256; ++b) {
         const float q = (float)(int8_t)b;
-        if (dtype == DT_BF16) { table_out[b] = kTables<DT_BF16>.v[256 + b]; arithmetic_out[b] = ecc_fraction<DT_BF16, 1>(q); }
-        else { table_out[b] = kTables<DT_F16>.v[256 + b]; arithmetic_out[b] = ecc_fraction<DT_F16, 1>(q); }
+        if (dtype == DT_BF16) { table_out[b] = kTables<DT_BF16>.v[256 * kTableEcc + b]; arithmetic_out[b] = ecc_fraction<DT_BF16, 1>(q); }
+        else { table_out[b] = kTables<DT_F16>.v[256 * kTableEcc + b]; arithmetic_out[b] = ecc_fraction<DT_F16, 1>(q); }
     }
 }
 // codes of one group from its first-moment values m and second-moment values v: through the quick forms with
@@ -311,7 +311,7 @@ int64_t hm_quantize_group_from_moments(const float* m, const float* v, int8_t* q
     }
     return failed;
 }
-void hm_softsign_table(float* out) { for (int b = 0; b < 256; ++b) out[b] = kTable.v[b]; }
+void hm_softsign_table(float* out) { for (int b = 0; b < 256; ++b) out[b] = kTable.v[256 * kTableMom + b]; }
 
 int hm_ecc_join(const void* narrow, int narrow_dtype, const void* ecc, int ecc_bytes, float* out, int64_t n) {
     for (int64_t i = 0; i < n; ++i) {
