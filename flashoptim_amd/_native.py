@@ -51,8 +51,11 @@ class FoChunk(ctypes.Structure):
     ]
 
 
+_DIAG_LIB_PATH = os.path.join(os.path.dirname(_LIB_PATH), "libflashoptim_hip_diag.so")
+
 _lock = threading.Lock()
 _lib: Optional[ctypes.CDLL] = None
+_diag_lib: Optional[ctypes.CDLL] = None
 
 # name -> (restype, argtypes); kept in one table so a test can check it against the header
 _vp, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
@@ -76,7 +79,10 @@ SIGNATURES = {
     "fo_dequantize": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp]),
     "fo_ecc_join": (_i32, [_vp, _i32, _vp, _i32, _vp, _i64, _vp]),
     "fo_ecc_split": (_i32, [_vp, _vp, _i32, _vp, _i32, _i64, _vp]),
-    # include/flashoptim_hip_diag.h
+}
+# include/flashoptim_hip_diag.h: exported by the diagnostics build only (libflashoptim_hip_diag.so, which also
+# exports everything above)
+DIAG_SIGNATURES = {
     "fo_copy_bytes": (_i32, [_vp, _vp, _i64, _vp]),
     "fo_multi_adam_streams_copy": (_i32, [_vp, _i64, _vp, _i64, _i32, _i32, _i32, _vp]),
     "fo_multi_momentum_streams_copy": (_i32, [_vp, _i64, _vp, _i64, _i32, _i32, _i32, _vp]),
@@ -89,36 +95,55 @@ def library_path() -> str:
     return _LIB_PATH
 
 
+def _load(path: str, signatures: dict) -> ctypes.CDLL:
+    if not os.path.exists(path):
+        raise RuntimeError(
+            f"{path} is missing: flashoptim_amd has no implementation without its HIP "
+            "library. Build it with `make -C flashoptim_amd/csrc` (or __graft_entry__.build())."
+        )
+    handle = ctypes.CDLL(path)
+    for name, (restype, argtypes) in signatures.items():
+        try:
+            fn = getattr(handle, name)
+        except AttributeError:
+            raise RuntimeError(
+                f"{path} does not export {name}: it was built from older sources. Rebuild it with "
+                "`make -C flashoptim_amd/csrc`."
+            ) from None
+        fn.restype = restype
+        fn.argtypes = argtypes
+    return handle
+
+
 def lib() -> ctypes.CDLL:
     """Load the HIP library once; raise loudly when it has not been built."""
     global _lib
     if _lib is None:
         with _lock:
             if _lib is None:
-                if not os.path.exists(_LIB_PATH):
-                    raise RuntimeError(
-                        f"{_LIB_PATH} is missing: flashoptim_amd has no implementation without its HIP "
-                        "library. Build it with `make -C flashoptim_amd/csrc` (or __graft_entry__.build())."
-                    )
-                handle = ctypes.CDLL(_LIB_PATH)
-                for name, (restype, argtypes) in SIGNATURES.items():
-                    try:
-                        fn = getattr(handle, name)
-                    except AttributeError:
-                        raise RuntimeError(
-                            f"{_LIB_PATH} does not export {name}: it was built from older sources. Rebuild it with "
-                            "`make -C flashoptim_amd/csrc`."
-                        ) from None
-                    fn.restype = restype
-                    fn.argtypes = argtypes
-                _lib = handle
+                _lib = _load(_LIB_PATH, SIGNATURES)
     return _lib
 
 
-def check(rc: int, what: str) -> None:
-    """Translate a non-zero native return code into RuntimeError with the library's message."""
+def diag_lib() -> ctypes.CDLL:
+    """The diagnostics build of the library (measurement kernels and residency queries, for the benchmark and the
+    tests; the optimizer path never loads it)."""
+    global _diag_lib
+    if _diag_lib is None:
+        with _lock:
+            if _diag_lib is None:
+                _diag_lib = _load(_DIAG_LIB_PATH, {**SIGNATURES, **DIAG_SIGNATURES})
+    return _diag_lib
+
+
+def diag_library_path() -> str:
+    return _DIAG_LIB_PATH
+
+
+def check(rc: int, what: str, library: Optional[ctypes.CDLL] = None) -> None:
+    """Translate a non-zero native return code into RuntimeError with the message of the library that returned it."""
     if rc != 0:
-        msg = lib().fo_last_error().decode("utf-8", "replace")
+        msg = (library or lib()).fo_last_error().decode("utf-8", "replace")
         raise RuntimeError(f"{what} failed (code {rc}): {msg}")
 
 

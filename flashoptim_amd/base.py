@@ -73,7 +73,8 @@ class _Bucket:
     plan: Optional[BucketPlan]        # multi-tensor tables; None for single-tensor buckets
     step_pool: Optional[torch.Tensor]  # 1-D CPU fp32 tensor whose elements ARE the bucket's `step` scalars (Adam), else None
     step_value: Optional[int]
-    step_views: Optional[list] = None  # the 0-dim views of step_pool that were stored as state[p]["step"]
+    step_views: Optional[list] = None  # the 0-dim views of step_pool that were stored as state[p]["step"] (kept alive)
+    step_view_ids: Optional[list] = None  # their id()s: one list comparison per step notices a replaced counter object
 
 
 @dataclass
@@ -449,7 +450,8 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
             for t in tensors:
                 t.grad = None  # the cache must not keep gradients alive
             buckets.append(_Bucket(key.kind, key.dtype, key.ecc_bytes, key.quantized, [p for p, _ in items], tensors,
-                                   plan, step_pool, scalars.get("step"), step_views))
+                                   plan, step_pool, scalars.get("step"), step_views,
+                                   None if step_views is None else list(map(id, step_views))))
         if cacheable and buckets:
             needed = None
             if self._check_numerics:
@@ -474,9 +476,8 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
                 # step number from them, and leave counters that no longer agree to the per-parameter path.  A
                 # counter OBJECT that was replaced (state[p]["step"] = tensor(0.)) no longer aliases the pool.
                 state = self.state
-                for p, view in zip(b.params, b.step_views):
-                    if state[p].get("step") is not view:
-                        return False
+                if [id(state[p].get("step")) for p in b.params] != b.step_view_ids:
+                    return False
                 lo, hi = torch.aminmax(b.step_pool)
                 lo = lo.item()
                 if lo != hi.item():

@@ -1,7 +1,9 @@
 // Fused Adam / AdamW step kernel for gfx950 and its C entry points (ref: /root/reference/flashoptim/
 // optimizers.py:2203-2438, cited as "ref:").
 #include "fo_step.h"
+#ifdef FO_DIAG
 #include "../../include/flashoptim_hip_diag.h"
+#endif
 
 #include <mutex>
 
@@ -171,6 +173,7 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT = AdamExact<D
 };
 
 
+#ifdef FO_DIAG
 // The Adam step's memory accesses without its arithmetic: every stream of the step is loaded and stored back
 // unchanged through the same load / store code, launch geometry and residency mechanism.  It shows what rate this
 // mix of seven loads and six stores per wavefront reaches on the device, next to the step kernels' own rate.
@@ -210,6 +213,8 @@ template <int DT, int ECCB, bool QUANT> struct AdamStreamsOp {
         }
     }
 };
+
+#endif  // FO_DIAG
 
 }  // namespace fo
 
@@ -408,6 +413,7 @@ int fo_multi_adam_step_static(const fo_tensor_desc* host_descs, int64_t n_tensor
     return dispatch_adam(dtype, ecc_bytes, quantized, decoupled, 0, L);
 }
 
+#ifdef FO_DIAG
 int fo_multi_adam_streams_copy(const fo_tensor_desc* descs, int64_t n_tensors, const fo_chunk* chunks, int64_t n_chunks,
                                int dtype, int ecc_bytes, int quantized, void* stream) {
     if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
@@ -421,5 +427,7 @@ int fo_adam_step_residency(int dtype, int ecc_bytes, int quantized, int decouple
     ResidencyQuery q{multi, target, achieved, dynamic_lds};
     return decoupled ? dispatch<AdamWOp>(dtype, ecc_bytes, quantized, q) : dispatch<AdamL2Op>(dtype, ecc_bytes, quantized, q);
 }
+
+#endif  // FO_DIAG
 
 }  // extern "C"

@@ -1,14 +1,17 @@
-// Library-wide pieces of libflashoptim_hip.so: error text, device queries, the host-side chunk-table builder
-// of the multi-tensor launcher and the calibration copy kernel.
+// Library-wide pieces of libflashoptim_hip.so: error text, device queries and the host-side chunk-table builder
+// of the multi-tensor launcher; in the diagnostics build (FO_DIAG) also the calibration copy kernel.
 #include "fo_device.h"
 #include "fo_host.h"
 #include "../../include/flashoptim_hip.h"
+#ifdef FO_DIAG
 #include "../../include/flashoptim_hip_diag.h"
+#endif
 
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
 
+#ifdef FO_DIAG
 namespace fo {
 
 constexpr int kCopyThreads = 64;
@@ -28,6 +31,7 @@ __global__ __launch_bounds__(kCopyThreads) void copy_kernel(u32x4* __restrict__ 
 
 
 }  // namespace fo
+#endif  // FO_DIAG
 
 namespace fo_host {
 
@@ -126,6 +130,7 @@ int64_t fo_build_chunks(const int64_t* numels, int64_t n_tensors, int tiles_per_
     return c;
 }
 
+#ifdef FO_DIAG
 int fo_copy_bytes(void* dst, const void* src, int64_t n_bytes, void* stream) {
     if (n_bytes < 0 || (n_bytes & 15)) return fail(FO_ERR_INVALID_ARGUMENT, "n_bytes must be a non-negative multiple of 16");
     if (n_bytes == 0) return 0;
@@ -139,5 +144,7 @@ int fo_copy_bytes(void* dst, const void* src, int64_t n_bytes, void* stream) {
                        (fo::u32x4*)dst, (const fo::u32x4*)src, n_vec, grid * fo::kCopyThreads, passes);
     return check_hip(hipGetLastError(), "copy kernel launch");
 }
+
+#endif  // FO_DIAG
 
 }  // extern "C"

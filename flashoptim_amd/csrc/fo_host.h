@@ -15,8 +15,11 @@ int check_hip(hipError_t e, const char* what);
 int compute_units();
 const char* last_error();
 
-// The library's one debug switch: FO_DEBUG_WG_PER_CU=<n> in the environment (read once) makes every step kernel
-// cap its residency at n workgroups per compute unit instead of its own measured optimum; 0 when unset.
+// The library's one debug switch: FO_DEBUG_WG_PER_CU=<n> in the environment (1..32, read once) makes every step
+// kernel ask for n resident workgroups per compute unit instead of its own measured optimum; 0 when unset.  What
+// results is the next count the LDS allocation units can enforce at or above n (fo_step.h: plan_residency; a launch
+// can request at most 64 KiB, so nothing below 3), further limited by a kernel's cap of wavefronts per SIMD; the
+// residency queries of the diagnostics build report it.
 int debug_workgroups_per_cu();
 
 // Shared argument check of the multi-tensor entry points: counts, dtype code and table pointers.

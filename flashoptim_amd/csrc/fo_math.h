@@ -250,6 +250,9 @@ FO_FN u32 quantize_var_code(float r, float av, float rav) { return (u32)(int)qua
 //     first moment   exact 3.8e-5, quick 3.8e-5   ->  they can differ by 7.6e-5   ->  margin 2^-13 = 1.2e-4
 //     second moment  exact 7.6e-5, quick 1.2e-4   ->  they can differ by 2.0e-4   ->  margin 2^-12 = 2.4e-4
 // so when the quick value lies farther than the margin from every integer, floor() of it IS the exact form's code.
+// Precondition: am + |m| and av stay below 2^126 (beyond that the reciprocal instruction returns a subnormal, flushed
+// to zero).  The group scale is stored as fp16 and overflows at 65504, forty orders of magnitude earlier, so a state
+// that large is already lost; the bound is stated, not enforced.
 // The margin is added up front (so the test is one fract and one compare: fract(x + margin) >= 2 margin) and a value
 // that fails the test is requantised with the exact form.  About 2.4e-4 of the first-moment and 4.9e-4 of the
 // second-moment values of a continuous distribution fail it; values that sit on a rounding boundary to the last bit

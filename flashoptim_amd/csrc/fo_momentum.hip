@@ -1,7 +1,9 @@
 // Fused SGD / SGDW / Nesterov / Lion step kernels (and the momentum-free SGD step) for gfx950 with their C
 // entry points (ref: /root/reference/flashoptim/optimizers.py:1447-1465, 1535-1719, cited as "ref:").
 #include "fo_step.h"
+#ifdef FO_DIAG
 #include "../../include/flashoptim_hip_diag.h"
+#endif
 
 namespace fo {
 
@@ -106,6 +108,7 @@ template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumOp {
 };
 
 
+#ifdef FO_DIAG
 // The momentum step's memory accesses without its arithmetic (see AdamStreamsOp in fo_adam.hip): parameters,
 // gradients, ECC, the moment's codes and scales are loaded and everything but the gradients is stored back unchanged
 // by the step's own load / store code.
@@ -137,6 +140,8 @@ template <int DT, int ECCB, bool QUANT> struct MomentumStreamsOp {
         }
     }
 };
+
+#endif  // FO_DIAG
 
 }  // namespace fo
 
@@ -189,6 +194,7 @@ int fo_multi_sgd_plain_step(const fo_tensor_desc* descs, int64_t n_tensors, cons
     return dispatch<PlainOp>(dtype, ecc_bytes, 0, L);
 }
 
+#ifdef FO_DIAG
 int fo_multi_momentum_streams_copy(const fo_tensor_desc* descs, int64_t n_tensors, const fo_chunk* chunks, int64_t n_chunks,
                                    int dtype, int ecc_bytes, int quantized, void* stream) {
     if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
@@ -204,5 +210,7 @@ int fo_momentum_step_residency(int dtype, int ecc_bytes, int quantized, int kind
     if (kind == fo::KIND_PLAIN) return dispatch<PlainOp>(dtype, ecc_bytes, 0, q);
     return dispatch<SgdOp>(dtype, ecc_bytes, quantized, q);
 }
+
+#endif  // FO_DIAG
 
 }  // extern "C"

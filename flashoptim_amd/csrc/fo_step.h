@@ -173,7 +173,7 @@ __device__ __forceinline__ void quantize_mom_var_quick_verified(const float (&m)
     const float least_m = fminf(fminf(slack_m[0], slack_m[1]), fminf(slack_m[2], slack_m[3]));
     const float least_v = fminf(fminf(slack_v[0], slack_v[1]), fminf(slack_v[2], slack_v[3]));
     convert_pack8<kFloor, kTrunc>(xm, xv, mout.w[0], vout.w[0]);
-    const bool any = !quick_slack_is_safe(least_m, kQuickMarginMom) | !quick_slack_is_safe(least_v, kQuickMarginVar);
+    const bool any = !quick_slack_is_safe(least_m, kQuickMarginMom) || !quick_slack_is_safe(least_v, kQuickMarginVar);
     if (__builtin_amdgcn_ballot_w64(any) != 0) {
         const float ram = hw::rcp(am), rav = hw::rcp(av_exact);
 #pragma unroll

@@ -364,5 +364,6 @@ def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
     if not src.is_contiguous() or not dst.is_contiguous():
         raise ValueError("copy_bytes needs contiguous tensors")
     with _native.device_guard(src.device):
-        rc = _native.lib().fo_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes, _native.current_stream_ptr(src.device))
-    _native.check(rc, "fo_copy_bytes")
+        diag = _native.diag_lib()
+        rc = diag.fo_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes, _native.current_stream_ptr(src.device))
+    _native.check(rc, "fo_copy_bytes", diag)

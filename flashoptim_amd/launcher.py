@@ -137,10 +137,12 @@ class BucketPlan:
         self.chunks_dev = host.to(self.device)
         nbytes = self.n_tensors * ctypes.sizeof(FoTensorDesc)
         self.descs_dev = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
-        # one pinned staging buffer for the life of the plan; `_staged` marks the last copy out of it
-        self._staging = torch.empty(nbytes, dtype=torch.uint8).pin_memory()
+        # two pinned staging buffers for the life of the plan, used in turn; `_staged[i]` marks the last copy out of
+        # buffer i
+        self._staging = [torch.empty(nbytes, dtype=torch.uint8).pin_memory() for _ in range(2)]
         self._table_bytes = torch.frombuffer(self.table, dtype=torch.uint8)  # a view of the ctypes table, no copy
-        self._staged: Optional[torch.cuda.Event] = None
+        self._staged: list[Optional[torch.cuda.Event]] = [None, None]
+        self._next_staging = 0
         self._dirty = True
 
     def set_grad_ptr(self, index: int, ptr: int) -> None:
@@ -155,14 +157,20 @@ class BucketPlan:
                 "uploaded again, which cannot be recorded into a HIP graph (a replay would copy whatever the staging "
                 "buffer holds by then). Run one step outside the capture with the gradient buffers the graph will use "
                 "(static gradients, zero_grad(set_to_none=False)), then capture.")
-        if self._staged is not None:
-            self._staged.synchronize()  # the previous upload has read the staging buffer (normally long ago)
-        self._staging.copy_(self._table_bytes)
+        # The host waits only when the copy out of this buffer, queued two uploads ago, has not run yet: with
+        # gradients that move every step the host can therefore run two iterations ahead of the device before it
+        # blocks here (a single buffer would tie it to the previous step's copy, which sits behind a whole iteration
+        # of queued work).
+        i = self._next_staging
+        self._next_staging = 1 - i
+        if self._staged[i] is not None and not self._staged[i].query():
+            self._staged[i].synchronize()
+        self._staging[i].copy_(self._table_bytes)
         # stream-ordered: launches already queued with the previous table finish before it is overwritten
-        self.descs_dev.copy_(self._staging, non_blocking=True)
-        if self._staged is None:
-            self._staged = torch.cuda.Event()
-        self._staged.record()
+        self.descs_dev.copy_(self._staging[i], non_blocking=True)
+        if self._staged[i] is None:
+            self._staged[i] = torch.cuda.Event()
+        self._staged[i].record()
         self._dirty = False
 
     def launch(self, **scalars) -> None:
@@ -190,9 +198,9 @@ class BucketPlan:
         _native.check(rc, "fo_multi_sgd_plain_step" if self.kind == "plain" else f"fo_multi_{self.kind}_step")
 
     def launch_streams_copy(self) -> None:
-        """Measurement aid (Adam and momentum buckets): read every stream of the bucket and write it back unchanged
-        with the step kernels' access code, without the step's arithmetic; shows what rate the step's access mix can
-        reach."""
+        """Measurement aid (Adam and momentum buckets; needs the diagnostics build of the library): read every stream
+        of the bucket and write it back unchanged with the step kernels' access code, without the step's arithmetic;
+        shows what rate the step's access mix can reach."""
         if self.kind not in ("adam", "momentum"):
             raise ValueError("the access-mix copy exists for Adam and momentum buckets only")
         if self.n_chunks == 0:
@@ -200,7 +208,8 @@ class BucketPlan:
         with _native.device_guard(self.device):
             if self._dirty:
                 self._upload()
-            entry = getattr(_native.lib(), f"fo_multi_{self.kind}_streams_copy")
+            diag = _native.diag_lib()
+            entry = getattr(diag, f"fo_multi_{self.kind}_streams_copy")
             rc = entry(self.descs_dev.data_ptr(), self.n_tensors, self.chunks_dev.data_ptr(), self.n_chunks,
                        DTYPE_CODE[self.dtype], self.ecc_bytes, int(self.quantized), _native.current_stream_ptr(self.device))
-        _native.check(rc, f"fo_multi_{self.kind}_streams_copy")
+        _native.check(rc, f"fo_multi_{self.kind}_streams_copy", diag)

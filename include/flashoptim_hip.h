@@ -130,6 +130,10 @@ int fo_multi_momentum_step(const fo_tensor_desc *descs, int64_t n_tensors, const
  * FO_STATIC_MAX_TENSORS tensors are refused; lists with more than FO_STATIC_MAX_CHUNKS tiles are covered with
  * several 4096-element tiles per work item.  Results are bit-identical to fo_multi_adam_step.  All calls on one
  * device share the one array: calls that overlap in time on a device (different streams or threads) race.
+ * The first call on a device, and the first call of each kernel variant (dtype, ecc_bytes, quantized, decoupled)
+ * there, takes the array's address and plans the kernel's residency through host API calls that must not run while
+ * the stream is capturing: make one eager call per variant before capturing.  After that a call enqueues kernel
+ * launches only.  There is no `_exact` twin of this entry point: it runs what fo_multi_adam_step runs.
  */
 #define FO_STATIC_MAX_TENSORS 1024
 #define FO_STATIC_MAX_CHUNKS 65536

@@ -1,8 +1,11 @@
 /*
- * flashoptim_hip_diag.h -- measurement and diagnostic entry points of libflashoptim_hip.so.
+ * flashoptim_hip_diag.h -- measurement and diagnostic entry points.
  *
  * Nothing here is part of the optimizer path and none of it has a counterpart in the reference
- * (/root/reference/flashoptim/optimizers.py): the symbols exist for the benchmark and the tests.
+ * (/root/reference/flashoptim/optimizers.py): the symbols exist for the benchmark and the tests.  They are exported by
+ * the diagnostics build of the library only (libflashoptim_hip_diag.so: the product's sources compiled with
+ * -DFO_DIAG, so it also exports everything in flashoptim_hip.h and its step kernels are the product's, from the same
+ * text with the same flags); libflashoptim_hip.so holds product kernels only.
  */
 #ifndef FLASHOPTIM_HIP_DIAG_H
 #define FLASHOPTIM_HIP_DIAG_H
@@ -37,8 +40,9 @@ int fo_multi_momentum_streams_copy(const fo_tensor_desc *descs, int64_t n_tensor
 
 /*
  * Residency plan of a step kernel on the current device: the workgroups per compute unit the kernel family asks
- * for (`target`), what the runtime's occupancy query reports for the dynamic LDS request that enforces it
- * (`achieved`) and that request in bytes (`dynamic_lds`).  Any output pointer may be NULL.
+ * for (`target`), what the dynamic LDS request that enforces it, the runtime's occupancy query and the kernel's cap
+ * of wavefronts per SIMD allow together (`achieved`) and that request in bytes (`dynamic_lds`).  Any output pointer
+ * may be NULL.
  *   multi: 0 = the single-tensor kernel, 1 = the multi-tensor kernel.
  *   kind (momentum): 0 = SGD / SGDW / Nesterov, 1 = Lion, 2 = momentum-free SGD.
  */

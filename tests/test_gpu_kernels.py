@@ -19,6 +19,11 @@ def _native_lib():
     return _native.lib()
 
 
+def _diag_lib():
+    from flashoptim_amd import _native
+    return _native.diag_lib()
+
+
 def _k():
     from flashoptim_amd import kernels
     return kernels
@@ -601,7 +606,7 @@ def test_step_kernels_are_resident_as_planned():
     intended residency for every kernel family, in both grid shapes."""
     import ctypes
 
-    lib = _native_lib()
+    lib = _diag_lib()  # the same sources and flags as the product library, plus the queries
     want_adam = {(0, 0): 18, (1, 0): 16, (1, 1): 16, (1, 2): 20, (2, 0): 16, (2, 1): 20, (2, 2): 20}
     for (dtype, ecc), want in want_adam.items():
         for quantized in (1, 0):

@@ -1258,3 +1258,80 @@ def test_rewritten_step_counters_are_honoured_by_the_cached_plan():
         for k in sa:
             assert parity.bits_equal(sa[k], sb[k]), k
     assert [float(oa.state[p]["step"]) for p in pa] == [5.0, 43.0, 5.0]
+
+
+class _ShardStub(nn.Parameter):
+    """What a sharding wrapper hands an optimizer: an object whose ``to_local()`` is this rank's shard
+    (/root/reference/flashoptim/optimizers.py:598-616).  Here the object's own storage is the shard."""
+
+    @staticmethod
+    def __new__(cls, data):
+        return torch.Tensor._make_subclass(cls, data, True)
+
+    def to_local(self):
+        self.calls = getattr(self, "calls", 0) + 1
+        return self.data
+
+
+@pytest.mark.parametrize("factory,kwargs", [
+    ("FlashAdamW", dict(lr=1e-3, weight_decay=0.01)),
+    ("FlashLion", dict(lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1)),
+])
+def test_a_tensor_stepped_as_shards_equals_the_whole_tensor(factory, kwargs):
+    """The path shards without any exchange: every 32-element quantisation group is independent and the update is
+    elementwise.  One bf16 tensor is stepped whole and as two shards that reach the optimizer through ``to_local()``
+    (ref:598-616, 724-730, 999-1001; state is created from the local shard).
+    Split at a multiple of 32 elements: parameters, correction codes, moment codes and group scales of the shards,
+    laid end to end, equal the whole tensor's bit for bit on every step.
+    Split anywhere else: the groups behind the split start at other elements, so their scales and codes are those
+    of other groups (which is why a compressed checkpoint is tied to its sharding); the first step, which starts
+    from zero states, still gives bit-identical parameters, and later steps stay as close as two quantisations of
+    the same moments do."""
+    fo = _fo()
+    n = 3 * 4096 + 777
+    torch.manual_seed(5)
+    w0 = (torch.randn(n, device=DEV) * 0.02).to(torch.bfloat16)
+    grads = [(torch.randn(n, device=DEV) * 1e-3).to(torch.bfloat16) for _ in range(4)]
+    names = [k for k in ("exp_avg", "exp_avg_sq") if factory == "FlashAdamW" or k == "exp_avg"]
+
+    def run(cuts):
+        """Steps the tensor cut at `cuts`; returns per step the pieces' outputs laid end to end."""
+        bounds = [0] + list(cuts) + [n]
+        params = [(_ShardStub if cuts else nn.Parameter)(w0[a:b].clone()) for a, b in zip(bounds, bounds[1:])]
+        opt = getattr(fo, factory)(params, master_weight_bits=24, **kwargs)
+        out = []
+        for g in grads:
+            for p, a, b in zip(params, bounds, bounds[1:]):
+                p.grad = g[a:b].clone()
+            opt.step()
+            rec = dict(p=torch.cat([p.detach().reshape(-1) for p in params]).clone(),
+                       ecc=torch.cat([opt.state[p]["error_bits"].reshape(-1) for p in params]).clone())
+            for k in names:
+                rec[k] = torch.cat([opt.state[p][k].quantized.reshape(-1) for p in params]).clone()
+                rec[k + "_scales"] = [opt.state[p][k].scales.clone() for p in params]
+            out.append(rec)
+        if cuts:
+            assert all(getattr(p, "calls", 0) > 0 for p in params), "the optimizer never asked for the local shard"
+            assert all(opt.state[p][names[0]].quantized.numel() == p.numel() for p in params)
+        return out
+
+    whole = run(())
+    aligned = run((4096 + 64,))
+    for step, (a, b) in enumerate(zip(whole, aligned), start=1):
+        for key in ("p", "ecc") + tuple(names):
+            assert parity.bits_equal(a[key], b[key]), f"aligned split, step {step}: {key} differs"
+        for k in names:
+            assert parity.bits_equal(a[k + "_scales"][0], torch.cat(b[k + "_scales"])), f"aligned split, step {step}: {k} scales differ"
+    ragged = run((4096 + 50,))
+    assert parity.bits_equal(whole[0]["p"], ragged[0]["p"]) and parity.bits_equal(whole[0]["ecc"], ragged[0]["ecc"])
+    cut = 4096 + 50
+    for step, (a, b) in enumerate(zip(whole, ragged), start=1):
+        # in front of the cut nothing changes; behind it only the grouping of the moments does
+        for key in ("p", "ecc") + tuple(names):
+            assert parity.bits_equal(a[key][:cut - cut % 32], b[key][:cut - cut % 32]), f"ragged split, step {step}: {key} differs before the cut"
+        pa, pb = a["p"].float(), b["p"].float()
+        # behind the cut the two runs dequantise slightly different moments: their updates (at most lr per step under
+        # Adam, exactly lr under Lion, whose sign may flip) drift apart by a fraction of what was applied
+        assert float((pa - pb).abs().max()) <= 2.0 * kwargs["lr"] * step, f"ragged split, step {step}"
+        assert float((pa - pb).abs().mean()) <= 0.05 * kwargs["lr"] * step, f"ragged split, step {step}"
+    assert not parity.bits_equal(whole[-1][names[0]], ragged[-1][names[0]])          # the groups behind the cut are other groups

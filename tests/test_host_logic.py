@@ -33,26 +33,34 @@ NO_GPU = not torch.cuda.is_available()
 # ------------------------------------------------------------------------------------------- C ABI
 
 
-HEADERS = ("flashoptim_hip.h", "flashoptim_hip_diag.h")   # the product ABI; measurement and diagnostic symbols
+def _declared_symbols(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fo_[a-z0-9_]+)\s*\(", text)))
 
 
-def _declared_symbols():
-    names = set()
-    for header in HEADERS:
-        text = open(os.path.join(ROOT, "include", header)).read()
-        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-        names.update(re.findall(r"\b(fo_[a-z0-9_]+)\s*\(", text))
-    return sorted(names)
+def _exported_symbols(path):
+    import subprocess
+
+    out = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True, check=True).stdout
+    return sorted(line.split()[-1] for line in out.splitlines() if line.split()[-1].startswith("fo_"))
 
 
 def test_library_exports_every_declared_symbol():
+    """The product library exports exactly what include/flashoptim_hip.h declares (no measurement kernels); the
+    diagnostics build exports that plus include/flashoptim_hip_diag.h; the ctypes tables bind exactly those."""
+    product, diag = _declared_symbols("flashoptim_hip.h"), _declared_symbols("flashoptim_hip_diag.h")
+    assert len(product) >= 15 and len(diag) >= 4 and not set(product) & set(diag)
     lib = _native.lib()
-    declared = _declared_symbols()
-    assert len(declared) >= 15
-    for name in declared:
-        assert hasattr(lib, name), f"{name} is declared in include/ but not exported"
-    # and the ctypes table binds exactly the declared entry points
-    assert sorted(_native.SIGNATURES) == declared
+    for name in product:
+        assert hasattr(lib, name), f"{name} is declared in include/flashoptim_hip.h but not exported"
+    assert _exported_symbols(_native.library_path()) == product
+    assert sorted(_native.SIGNATURES) == product
+    dlib = _native.diag_lib()
+    for name in product + diag:
+        assert hasattr(dlib, name), f"{name} is missing from the diagnostics build"
+    assert _exported_symbols(_native.diag_library_path()) == sorted(product + diag)
+    assert sorted(_native.DIAG_SIGNATURES) == diag
 
 
 def test_version_and_error_text_without_a_device():
@@ -69,7 +77,7 @@ def test_version_and_error_text_without_a_device():
     assert lib.fo_adam_step(None, None, None, None, None, None, None, 0, 1, 1, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, 1, None) == 0
     with pytest.raises(RuntimeError, match="code -1"):
         _native.check(-1, "fo_adam_step")
-    assert lib.fo_copy_bytes(None, None, 24, None) == -1
+    assert _native.diag_lib().fo_copy_bytes(None, None, 24, None) == -1
     assert lib.fo_ecc_join(None, 0, None, 1, None, 4, None) == -1  # fp32 "narrow" dtype is rejected
     assert lib.fo_ecc_split(None, None, 1, None, 3, 4, None) == -1
 

@@ -84,3 +84,36 @@ def test_more_tiles_than_chunk_entries_and_too_many_tensors():
     rc = _static_step(tiny, torch.bfloat16, 1, 1)
     assert rc != 0 and b"exceed" in _native.lib().fo_last_error()
     assert _static_step([], torch.bfloat16, 1, 1) == 0
+
+
+@pytest.mark.parametrize("dtype,ecc_dtype", [(torch.bfloat16, torch.int8), (torch.bfloat16, torch.int16)])
+def test_a_captured_static_call_replays_like_the_eager_entry_point(dtype, ecc_dtype):
+    """The callers this entry point is for include code under HIP graph capture.  The first call on a device (and
+    the first of each kernel variant) takes the address of the static array and plans the residency through host
+    API calls that must not run while a stream captures, so one eager call comes first.  After that a call records
+    nothing but kernel launches (the table-staging kernels and the step kernel; no copies, no memsets, no
+    allocation).  The step number travels by value, so every replay repeats the captured step number: each replay,
+    with new gradient values in the same buffers and eager work and synchronisations in between, must equal an
+    eager fo_multi_adam_step call with that step number, bit for bit."""
+    ecc_bytes = torch.empty(0, dtype=ecc_dtype).element_size()
+    lens = [1, 33, 4096, 70001, 12345] + [777] * 50
+    a, b = _make(lens, dtype, ecc_dtype, 11), _make(lens, dtype, ecc_dtype, 11)
+    plan = BucketPlan("adam", dtype, ecc_bytes, True, b)
+    _native.check(_static_step(a, dtype, ecc_bytes, 1), "fo_multi_adam_step_static")   # eager: set-up happens here
+    plan.launch(step=1, **HP)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = _static_step(a, dtype, ecc_bytes, 2)
+    _native.check(rc, "fo_multi_adam_step_static under capture")
+    gen = torch.Generator().manual_seed(12)
+    for replay in range(4):
+        for x, y in zip(a, b):   # new gradient values, same buffers
+            g = (torch.randn(x.grad.numel(), generator=gen) * 1e-3).to(dtype).to(DEV)
+            x.grad.copy_(g)
+            y.grad.copy_(g)
+        torch.cuda.synchronize()
+        graph.replay()
+        plan.launch(step=2, **HP)
+        torch.cuda.synchronize()
+        _same(a, b)
