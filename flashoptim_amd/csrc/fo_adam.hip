@@ -137,30 +137,16 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT = AdamExact<D
     using Hyper = AdamHyper;
     static constexpr int kLutMask = (QUANT ? 1 << kTableMom : 0) | (ECCB == 1 ? 1 << kTableEcc : 0);  // LDS code tables
     static constexpr int kDtype = DT;
-    // measured on MI355X with the 8B-parameter step and this file's ILP-oriented instruction schedule, over the
-    // residencies the LDS units allow (fo_step.h): 16 for 2-byte parameters (3.6-4.6 KiB of loads per wavefront; 14
-    // and 18 are two to three points worse on the 8B list), 18 for fp32 parameters (2.5 KiB per wavefront), 20 for
-    // the arithmetic-bound operation-by-operation update on 2-byte parameters.
-    // Wavefronts per SIMD: left alone, a compute unit spreads its sixteen wavefronts unevenly over the SIMDs on most
-    // boxes of the pool.  A cap of four (an even spread) gains 0.6 points there with 0- and 1-byte ECC and costs
-    // nothing on the other boxes.  With 2-byte ECC it gains two points on the former and loses 1.5 on the latter, and
-    // a cap of five is as erratic, so that variant stays uncapped, like fp32 (a cap costs a point there).  The
-    // operation-by-operation update on 2-byte parameters gains two points from its cap of five on every box.
+    // Measured on MI355X with the 8B-parameter step and this file's ILP-oriented instruction schedule, over the
+    // residencies the LDS units allow (fo_step.h):
+    //   guarded folded update on 2-byte parameters: 16 workgroups per compute unit, at most four wavefronts per SIMD
+    //     (14: -4 points, 18 with five per SIMD: -5, 21 with six: -6; 16 without the cap per SIMD: -0.4);
+    //   operation-by-operation update on 2-byte parameters (2-byte ECC, fp16 with a 1-byte ECC, the *_exact entry
+    //     points): 20 with at most five per SIMD (16/4: -3.5 points, 18/5 and 21/6: -1.3, 25 and 32 uncapped: -3);
+    //   fp32 parameters (2.5 KiB of loads per wavefront): 18, no cap (a cap costs a point).
     static constexpr bool kNarrowExact = EXACT && DT != DT_F32;
-#ifndef FO_EXACT_WG
-#define FO_EXACT_WG 20
-#endif
-#ifndef FO_EXACT_WAVES
-#define FO_EXACT_WAVES 5
-#endif
-#ifndef FO_FOLDED_WG
-#define FO_FOLDED_WG 16
-#endif
-#ifndef FO_FOLDED_WAVES
-#define FO_FOLDED_WAVES 4
-#endif
-    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 18 : (kNarrowExact ? FO_EXACT_WG : FO_FOLDED_WG);
-    static constexpr int kMaxWavesPerSimd = DT == DT_F32 ? 8 : (kNarrowExact ? FO_EXACT_WAVES : FO_FOLDED_WAVES);
+    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 18 : (kNarrowExact ? 20 : 16);
+    static constexpr int kMaxWavesPerSimd = DT == DT_F32 ? 8 : (kNarrowExact ? 5 : 4);
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
     template <int FAST> __device__ __forceinline__ static void load(const TensorPtrs& t, Where w, Raw& r) {
