@@ -38,6 +38,19 @@ __device__ __forceinline__ void adam_load(const TensorPtrs& t, Where w, AdamRaw<
     }
 }
 
+// Lane state of adam_redo_flagged (fo_math.h): the old weight is still in the lane's raw parameter and ECC words.
+template <int DT, int ECCB, bool QUANT> struct AdamRedoLane {
+    static constexpr int EPL = DTypeInfo<DT>::epl;
+    float (&p)[EPL];
+    const float (&slack)[EPL];
+    const float (&m)[EPL];
+    const float (&v)[EPL];
+    const AdamRaw<DT, ECCB, QUANT>& raw;
+    const float* lut;
+    float least;
+    __device__ __forceinline__ float old_master(int k) const { return master_of<DT, ECCB, EPL>(raw.p, raw.e, k, lut); }
+};
+
 template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT, int FAST>
 __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRaw<DT, ECCB, QUANT>& raw,
                                             const AdamHyper& h, const float* lut) {
@@ -75,23 +88,11 @@ __device__ __forceinline__ void adam_finish(const TensorPtrs& t, Where w, AdamRa
         m[k] = mn; r[k] = rk; v[k] = vn;
     }
     if constexpr (!EXACT) {
-        // The flagged elements again, operation by operation.  A wavefront with no flagged element branches past
-        // this; otherwise only the element positions that are flagged in some lane are redone.
-        float least = slack[0];
-#pragma unroll
-        for (int k = 1; k < EPL; ++k) least = fminf(least, slack[k]);
-        if (__builtin_amdgcn_ballot_w64(adam_folded_is_flagged(least)) != 0) {
-#pragma unroll
-            for (int k = 0; k < EPL; ++k) {
-                const bool redo = adam_folded_is_flagged(slack[k]);
-                if (__builtin_amdgcn_ballot_w64(redo) != 0) {
-                    float pk = master_of<DT, ECCB, EPL>(raw.p, raw.e, k, lut);
-                    if constexpr (DECOUPLED) pk = pk * h.one_m_wd;
-                    const float pe = adam_apply_exact(pk, m[k], v[k], h);
-                    if (redo) p[k] = pe;
-                }
-            }
-        }
+        // The flagged elements again, operation by operation (fo_math.h: adam_redo_flagged).  A wavefront with no
+        // flagged element branches past this; otherwise only the positions flagged in some lane are redone.
+        AdamRedoLane<DT, ECCB, QUANT> lane{p, slack, m, v, raw, lut};
+        HwWave<AdamRedoLane<DT, ECCB, QUANT>> wave{lane};
+        adam_redo_flagged<EPL, DECOUPLED>(wave, h);
     }
 
     Pack<ECCB, EPL> eout;

@@ -24,9 +24,15 @@
 #ifdef FO_MATH_HOST
 #include <math.h>
 #define FO_FN static inline
+#define FO_LANE_FN inline
+#define FO_LANE_ATTR
+#define FO_UNROLL
 #else
 #include <hip/hip_runtime.h>
 #define FO_FN __device__ __forceinline__
+#define FO_LANE_FN __device__ __forceinline__
+#define FO_LANE_ATTR __attribute__((always_inline))
+#define FO_UNROLL _Pragma("unroll")
 #endif
 
 namespace fo {
@@ -410,6 +416,144 @@ FO_FN float adam_apply_folded(float p, float mn, float r, const AdamHyper& h, fl
     return pn;
 }
 FO_FN bool adam_folded_is_flagged(float slack) { return slack < 0.0f; }
+
+// ------------------------------------------------------------------------------------------------
+// wave-level control flow of the verified forms
+// ------------------------------------------------------------------------------------------------
+// The verified forms act on a whole wavefront.  Every lane converts its values from the quick forms and keeps each
+// value's slack; the wavefront asks once whether any lane holds a value that failed its test (most wavefronts branch
+// past the repair there), and only then looks at the element positions one by one: a position is recomputed with
+// the exact form -- by every lane, the result kept by the lanes in which it failed -- only if it failed in some lane.
+// The flows are written once, over a `Wave`:
+//     wave.each(f)   runs f(lane) for every lane of the wavefront,
+//     wave.any(p)    tells whether p(lane) holds in some lane,
+// with `lane` the lane's own state (the structs named below).  In the kernels a Wave is the hardware wavefront seen
+// from one of its lanes (each: one call; any: a ballot; fo_step.h) and the lane state lives in registers; in the CPU
+// build used by the tests it is an array of 64 lane states (each: a loop; any: a logical or), so the same text runs
+// with a chosen lane and position failing.
+
+// Requantisation of a lane's N first-moment values.  Lane members:
+//   m[N], am            the values and the group absmax (clamped at 1e-12)
+//   x[N], slack[N], least, ram    scratch of the flow
+//   convert_mom(x)      codes of all N values from their quick values (floor)
+//   set_mom_code(k, c)  replaces the code of position k
+template <int N, class Wave> FO_FN void requantize_mom_verified(Wave& wave) {
+    wave.each([](auto& L) FO_LANE_ATTR {
+        FO_UNROLL for (int k = 0; k < N; ++k) {
+            L.x[k] = quantize_mom_quick(L.m[k], L.am);
+            L.slack[k] = quick_value_slack(L.x[k]);
+        }
+        L.least = L.slack[0];
+        FO_UNROLL for (int k = 1; k < N; ++k) L.least = fminf(L.least, L.slack[k]);
+        L.convert_mom(L.x);
+    });
+    if (wave.any([](const auto& L) FO_LANE_ATTR { return !quick_slack_is_safe(L.least, kQuickMarginMom); })) {
+        wave.each([](auto& L) FO_LANE_ATTR { L.ram = hw::rcp(L.am); });
+        FO_UNROLL for (int k = 0; k < N; ++k) {
+            if (wave.any([k](const auto& L) FO_LANE_ATTR { return !quick_slack_is_safe(L.slack[k], kQuickMarginMom); })) {
+                wave.each([k](auto& L) FO_LANE_ATTR {
+                    const u32 code = quantize_mom_code(L.m[k], L.am, L.ram);
+                    if (!quick_slack_is_safe(L.slack[k], kQuickMarginMom)) L.set_mom_code(k, code);
+                });
+            }
+        }
+    }
+}
+
+// Requantisation of a lane's N second-moment values.  Lane members:
+//   v[N], r[N]          the values and hw::sqrt of them
+//   av_quick, av        hw::sqrt and sqrt_corrected of the group's largest v (clamped at 1e-12)
+//   x[N], slack[N], least, rav    scratch of the flow
+//   convert_var(x), set_var_code(k, c)
+template <int N, class Wave> FO_FN void requantize_var_verified(Wave& wave) {
+    wave.each([](auto& L) FO_LANE_ATTR {
+        const float rav255 = hw::rcp(L.av_quick) * 255.0f;
+        FO_UNROLL for (int k = 0; k < N; ++k) {
+            L.x[k] = quantize_var_quick(L.r[k], rav255);
+            L.slack[k] = quick_value_slack(L.x[k]);
+        }
+        L.least = L.slack[0];
+        FO_UNROLL for (int k = 1; k < N; ++k) L.least = fminf(L.least, L.slack[k]);
+        L.convert_var(L.x);
+    });
+    if (wave.any([](const auto& L) FO_LANE_ATTR { return !quick_slack_is_safe(L.least, kQuickMarginVar); })) {
+        wave.each([](auto& L) FO_LANE_ATTR { L.rav = hw::rcp(L.av); });
+        FO_UNROLL for (int k = 0; k < N; ++k) {
+            if (wave.any([k](const auto& L) FO_LANE_ATTR { return !quick_slack_is_safe(L.slack[k], kQuickMarginVar); })) {
+                wave.each([k](auto& L) FO_LANE_ATTR {
+                    const u32 code = quantize_var_code(sqrt_corrected(L.v[k]), L.av, L.rav);
+                    if (!quick_slack_is_safe(L.slack[k], kQuickMarginVar)) L.set_var_code(k, code);
+                });
+            }
+        }
+    }
+}
+
+// Both moments of a lane that holds N values of each (fp32 parameters, N = 4): one conversion, one repair branch.
+// Lane members: those of the two flows above with the scratch doubled (xm, xv, slack_m, slack_v, least_m, least_v)
+// and convert_both(xm, xv).
+template <int N, class Wave> FO_FN void requantize_both_verified(Wave& wave) {
+    wave.each([](auto& L) FO_LANE_ATTR {
+        const float rav255 = hw::rcp(L.av_quick) * 255.0f;
+        FO_UNROLL for (int k = 0; k < N; ++k) {
+            L.xm[k] = quantize_mom_quick(L.m[k], L.am);
+            L.xv[k] = quantize_var_quick(L.r[k], rav255);
+            L.slack_m[k] = quick_value_slack(L.xm[k]);
+            L.slack_v[k] = quick_value_slack(L.xv[k]);
+        }
+        L.least_m = L.slack_m[0];
+        L.least_v = L.slack_v[0];
+        FO_UNROLL for (int k = 1; k < N; ++k) {
+            L.least_m = fminf(L.least_m, L.slack_m[k]);
+            L.least_v = fminf(L.least_v, L.slack_v[k]);
+        }
+        L.convert_both(L.xm, L.xv);
+    });
+    if (wave.any([](const auto& L) FO_LANE_ATTR {
+            return !quick_slack_is_safe(L.least_m, kQuickMarginMom) || !quick_slack_is_safe(L.least_v, kQuickMarginVar);
+        })) {
+        wave.each([](auto& L) FO_LANE_ATTR { L.ram = hw::rcp(L.am); L.rav = hw::rcp(L.av); });
+        FO_UNROLL for (int k = 0; k < N; ++k) {
+            if (wave.any([k](const auto& L) FO_LANE_ATTR { return !quick_slack_is_safe(L.slack_m[k], kQuickMarginMom); })) {
+                wave.each([k](auto& L) FO_LANE_ATTR {
+                    const u32 code = quantize_mom_code(L.m[k], L.am, L.ram);
+                    if (!quick_slack_is_safe(L.slack_m[k], kQuickMarginMom)) L.set_mom_code(k, code);
+                });
+            }
+            if (wave.any([k](const auto& L) FO_LANE_ATTR { return !quick_slack_is_safe(L.slack_v[k], kQuickMarginVar); })) {
+                wave.each([k](auto& L) FO_LANE_ATTR {
+                    const u32 code = quantize_var_code(sqrt_corrected(L.v[k]), L.av, L.rav);
+                    if (!quick_slack_is_safe(L.slack_v[k], kQuickMarginVar)) L.set_var_code(k, code);
+                });
+            }
+        }
+    }
+}
+
+// The repair of the guarded folded Adam update: the positions flagged in some lane again, operation by operation.
+// Lane members:
+//   p[N]                the folded results, overwritten where flagged
+//   slack[N]            from adam_apply_folded (negative = flagged); least: scratch
+//   m[N], v[N]          the new moments
+//   old_master(k)       the weight before the step (fp32 master, before the decoupled decay)
+template <int N, bool DECOUPLED, class Wave> FO_FN void adam_redo_flagged(Wave& wave, const AdamHyper& h) {
+    wave.each([](auto& L) FO_LANE_ATTR {
+        L.least = L.slack[0];
+        FO_UNROLL for (int k = 1; k < N; ++k) L.least = fminf(L.least, L.slack[k]);
+    });
+    if (wave.any([](const auto& L) FO_LANE_ATTR { return adam_folded_is_flagged(L.least); })) {
+        FO_UNROLL for (int k = 0; k < N; ++k) {
+            if (wave.any([k](const auto& L) FO_LANE_ATTR { return adam_folded_is_flagged(L.slack[k]); })) {
+                wave.each([k, &h](auto& L) FO_LANE_ATTR {
+                    float pk = L.old_master(k);
+                    if (DECOUPLED) pk = pk * h.one_m_wd;                                // ref:2363-2364
+                    const float pe = adam_apply_exact(pk, L.m[k], L.v[k], h);           // ref:2368-2375
+                    if (adam_folded_is_flagged(L.slack[k])) L.p[k] = pe;
+                });
+            }
+        }
+    }
+}
 
 // ------------------------------------------------------------------------------------------------
 // SGD / SGDW / Nesterov / Lion element update (ref:1624-1683, 1447-1465)

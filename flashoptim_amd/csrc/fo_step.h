@@ -96,100 +96,84 @@ template <int EPL> __device__ __forceinline__ void set_code(Pack<1, EPL>& out, i
     w = (w & ~(0xffu << sh)) | ((code & 0xffu) << sh);
 }
 
+// The hardware wavefront as the verified flows of fo_math.h see it from one of its lanes: each() is one call on the
+// lane's own state, any() a ballot over the 64 lanes.
+template <class Lane> struct HwWave {
+    Lane& lane;
+    template <class F> __device__ __forceinline__ void each(F&& f) { f(lane); }
+    template <class P> __device__ __forceinline__ bool any(P&& p) { return __builtin_amdgcn_ballot_w64(p(lane)) != 0; }
+};
+
+// Lane state of requantize_mom_verified / requantize_var_verified for eight values per lane (2-byte parameters):
+// the codes are the two dwords that travel to memory; the conversion writes each byte in place (convert_pack8).
+struct MomLane8 {
+    const float (&m)[8];
+    float am;
+    Pack<1, 8>& out;
+    float x[8], slack[8], least, ram;
+    __device__ __forceinline__ void convert_mom(const float (&q)[8]) {
+        const float lo[4] = {q[0], q[1], q[2], q[3]}, hi[4] = {q[4], q[5], q[6], q[7]};
+        convert_pack8<kFloor, kFloor>(lo, hi, out.w[0], out.w[1]);
+    }
+    __device__ __forceinline__ void set_mom_code(int k, u32 code) { set_code<8>(out, k, code); }
+};
+struct VarLane8 {
+    const float (&v)[8];
+    const float (&r)[8];
+    float av_quick, av;
+    Pack<1, 8>& out;
+    float x[8], slack[8], least, rav;
+    __device__ __forceinline__ void convert_var(const float (&q)[8]) {
+        const float lo[4] = {q[0], q[1], q[2], q[3]}, hi[4] = {q[4], q[5], q[6], q[7]};
+        convert_pack8<kTrunc, kTrunc>(lo, hi, out.w[0], out.w[1]);
+    }
+    __device__ __forceinline__ void set_var_code(int k, u32 code) { set_code<8>(out, k, code); }
+};
+// Four values of each moment per lane (fp32 parameters): one dword of codes per state, one conversion block.
+struct BothLane4 {
+    const float (&m)[4];
+    float am;
+    const float (&v)[4];
+    const float (&r)[4];
+    float av_quick, av;
+    Pack<1, 4>& mout;
+    Pack<1, 4>& vout;
+    float xm[4], xv[4], slack_m[4], slack_v[4], least_m, least_v, ram, rav;
+    __device__ __forceinline__ void convert_both(const float (&qm)[4], const float (&qv)[4]) {
+        convert_pack8<kFloor, kTrunc>(qm, qv, mout.w[0], vout.w[0]);
+    }
+    __device__ __forceinline__ void set_mom_code(int k, u32 code) { set_code<4>(mout, k, code); }
+    __device__ __forceinline__ void set_var_code(int k, u32 code) { set_code<4>(vout, k, code); }
+};
+
 // Quantises the lane's first-moment values against the group absmax `am` (shared by the group's lanes, clamped
-// at 1e-12); the rounding is the reference's (fo_math.h; ref:2405-2419, 1703-1710).  Through the quick forms:
-// every value is converted from its quick form; the values that fail the margin test are redone with the exact form.  A wavefront with no failing value (about four in five on
-// continuous data) branches past the repair; otherwise only the element positions k that failed in some lane are
-// redone.  The result is the exact requantiser's, code for code.
+// at 1e-12); the rounding is the reference's (fo_math.h; ref:2405-2419, 1703-1710).  Through the quick forms,
+// every value verified and the failing ones redone with the exact form (fo_math.h: requantize_mom_verified): the
+// result is the exact requantiser's, code for code.
 template <int EPL>
 __device__ __forceinline__ void quantize_mom_quick_verified(const float (&m)[EPL], float am, Pack<1, EPL>& out) {
     static_assert(EPL == 8, "two dwords of codes per lane");
-    float x[8], slack[8];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-        x[k] = quantize_mom_quick(m[k], am);
-        slack[k] = quick_value_slack(x[k]);
-    }
-    float least = slack[0];
-#pragma unroll
-    for (int k = 1; k < 8; ++k) least = fminf(least, slack[k]);
-    const float lo[4] = {x[0], x[1], x[2], x[3]}, hi[4] = {x[4], x[5], x[6], x[7]};
-    convert_pack8<kFloor, kFloor>(lo, hi, out.w[0], out.w[1]);
-    if (__builtin_amdgcn_ballot_w64(!quick_slack_is_safe(least, kQuickMarginMom)) != 0) {
-        const float ram = hw::rcp(am);
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const bool redo = !quick_slack_is_safe(slack[k], kQuickMarginMom);
-            if (__builtin_amdgcn_ballot_w64(redo) != 0) {
-                const u32 code = quantize_mom_code(m[k], am, ram);
-                if (redo) set_code<EPL>(out, k, code);
-            }
-        }
-    }
+    MomLane8 lane{m, am, out};
+    HwWave<MomLane8> wave{lane};
+    requantize_mom_verified<8>(wave);
 }
 // r: hw::sqrt of the lane's second moments v; av_quick / av_exact: hw::sqrt and sqrt_corrected of the group's largest v.
 template <int EPL>
 __device__ __forceinline__ void quantize_var_quick_verified(const float (&v)[EPL], const float (&r)[EPL], float av_quick,
                                                             float av_exact, Pack<1, EPL>& out) {
     static_assert(EPL == 8, "two dwords of codes per lane");
-    const float rav255 = hw::rcp(av_quick) * 255.0f;
-    float x[8], slack[8];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-        x[k] = quantize_var_quick(r[k], rav255);
-        slack[k] = quick_value_slack(x[k]);
-    }
-    float least = slack[0];
-#pragma unroll
-    for (int k = 1; k < 8; ++k) least = fminf(least, slack[k]);
-    const float lo[4] = {x[0], x[1], x[2], x[3]}, hi[4] = {x[4], x[5], x[6], x[7]};
-    convert_pack8<kTrunc, kTrunc>(lo, hi, out.w[0], out.w[1]);
-    if (__builtin_amdgcn_ballot_w64(!quick_slack_is_safe(least, kQuickMarginVar)) != 0) {
-        const float rav = hw::rcp(av_exact);
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const bool redo = !quick_slack_is_safe(slack[k], kQuickMarginVar);
-            if (__builtin_amdgcn_ballot_w64(redo) != 0) {
-                const u32 code = quantize_var_code(sqrt_corrected(v[k]), av_exact, rav);
-                if (redo) set_code<EPL>(out, k, code);
-            }
-        }
-    }
+    VarLane8 lane{v, r, av_quick, av_exact, out};
+    HwWave<VarLane8> wave{lane};
+    requantize_var_verified<8>(wave);
 }
 // Four elements per lane (fp32 parameters), both states through the quick forms with verification: one conversion
 // block, one repair branch.
 __device__ __forceinline__ void quantize_mom_var_quick_verified(const float (&m)[4], float am, const float (&v)[4],
                                                                 const float (&r)[4], float av_quick, float av_exact,
                                                                 Pack<1, 4>& mout, Pack<1, 4>& vout) {
-    const float rav255 = hw::rcp(av_quick) * 255.0f;
-    float xm[4], xv[4], slack_m[4], slack_v[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        xm[k] = quantize_mom_quick(m[k], am);
-        xv[k] = quantize_var_quick(r[k], rav255);
-        slack_m[k] = quick_value_slack(xm[k]);
-        slack_v[k] = quick_value_slack(xv[k]);
-    }
-    const float least_m = fminf(fminf(slack_m[0], slack_m[1]), fminf(slack_m[2], slack_m[3]));
-    const float least_v = fminf(fminf(slack_v[0], slack_v[1]), fminf(slack_v[2], slack_v[3]));
-    convert_pack8<kFloor, kTrunc>(xm, xv, mout.w[0], vout.w[0]);
-    const bool any = !quick_slack_is_safe(least_m, kQuickMarginMom) || !quick_slack_is_safe(least_v, kQuickMarginVar);
-    if (__builtin_amdgcn_ballot_w64(any) != 0) {
-        const float ram = hw::rcp(am), rav = hw::rcp(av_exact);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const bool redo_m = !quick_slack_is_safe(slack_m[k], kQuickMarginMom);
-            const bool redo_v = !quick_slack_is_safe(slack_v[k], kQuickMarginVar);
-            if (__builtin_amdgcn_ballot_w64(redo_m) != 0) {
-                const u32 code = quantize_mom_code(m[k], am, ram);
-                if (redo_m) set_code<4>(mout, k, code);
-            }
-            if (__builtin_amdgcn_ballot_w64(redo_v) != 0) {
-                const u32 code = quantize_var_code(sqrt_corrected(v[k]), av_exact, rav);
-                if (redo_v) set_code<4>(vout, k, code);
-            }
-        }
-    }
+    BothLane4 lane{m, am, v, r, av_quick, av_exact, mout, vout};
+    HwWave<BothLane4> wave{lane};
+    requantize_both_verified<4>(wave);
 }
 // Four elements per lane, one state (momentum kernels on fp32 parameters): plain conversion and byte packing.
 __device__ __forceinline__ void quantize_mom(const float (&m)[4], float am, Pack<1, 4>& out) {

@@ -40,6 +40,10 @@ def lib() -> ctypes.CDLL:
         L.hm_adam_step.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, f, f, f, f, f, i32, i32, i32, ctypes.POINTER(i64)]
         L.hm_adam_folded_update.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, f, f, f, f, f, i32, i32, vp, vp]
         L.hm_adam_folded_update.restype = None
+        L.hm_flow_stats.argtypes = [vp, i32]
+        L.hm_flow_stats.restype = None
+        L.hm_requantize_wave.argtypes = [vp] * 6
+        L.hm_requantize_wave.restype = None
         L.hm_code_over_255.argtypes = [vp]
         L.hm_code_over_255.restype = None
         L.hm_momentum_step.argtypes = [vp, vp, vp, vp, vp, i64, i32, i32, i32, f, f, f, f, i32, i32, i32]
@@ -102,6 +106,25 @@ def adam_folded_update(param, ecc, grad, mom, mom_scales, var, var_scales, lr, b
     lib().hm_adam_folded_update(_ptr(mom), _ptr(mom_scales), _ptr(var), _ptr(var_scales), _ptr(param), _ptr(grad), _ptr(ecc), n,
                                 lr, beta1, beta2, eps, weight_decay, int(decoupled), int(step), out.data_ptr(), redo.data_ptr())
     return out, redo.bool()
+
+
+def flow_stats(reset: bool = True) -> dict:
+    """What the simulated wavefronts did since the last reset: wavefronts stepped, wave-level questions asked
+    (one per verified flow and wavefront, plus one per element position once a flow repairs), how many were answered
+    with yes, and how many codes the repairs replaced."""
+    out = torch.zeros(4, dtype=torch.int64)
+    lib().hm_flow_stats(out.data_ptr(), int(reset))
+    return dict(zip(("waves", "questions", "yes", "codes_replaced"), out.tolist()))
+
+
+def requantize_wave(m: torch.Tensor, v: torch.Tensor):
+    """One wavefront (512 first-moment and 512 second-moment values, lane l holding values 8l .. 8l+7, four lanes per
+    quantisation group) through the kernels' verified requantisation flows.  Returns (codes of m, codes of v, the
+    exact forms' codes of m, of v)."""
+    assert m.numel() == 512 and v.numel() == 512 and m.dtype == v.dtype == torch.float32
+    out = [torch.empty(512, dtype=torch.uint8) for _ in range(4)]
+    lib().hm_requantize_wave(_ptr(m.contiguous()), _ptr(v.contiguous()), *(t.data_ptr() for t in out))
+    return out
 
 
 def code_over_255() -> torch.Tensor:

@@ -81,94 +81,226 @@ template <int DT, int ECCB> void write_master(void* param, void* ecc, int64_t i,
     if constexpr (ECCB > 0) store_ecc<ECCB>(ecc, i, ecc_split_bits<DT, ECCB, false>(p, w));
 }
 
-// the structure of adam_finish (fo_adam.hip), one quantisation group at a time.  `flagged` (may be null) counts the
-// elements whose folded update was redone operation by operation.
-template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT>
-void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scales, void* param, const void* grad, void* ecc,
-                 int64_t n, const AdamHyper& h, int64_t* flagged) {
-    for (int64_t g0 = 0; g0 < n; g0 += kGroup) {
-        const int cnt = (int)((n - g0) < kGroup ? (n - g0) : kGroup);
-        const int64_t group = g0 >> 5;
-        float sm = 1.0f, sv = 1.0f;
-        if (QUANT) { sm = f16_to_f32(mom_scales[group]); sv = f16_to_f32(var_scales[group]); }
-        float m[kGroup], v[kGroup];
-        float am = 0.0f, vmax = 0.0f;
-        for (int k = 0; k < cnt; ++k) {
-            const int64_t i = g0 + k;
-            const float p0 = read_master<DT, ECCB>(param, ecc, i);
-            float gr = load_elem<DT>(grad, i);
-            if (!DECOUPLED) gr = gr + p0 * h.wd;
-            float mn, vn;
-            if (QUANT) {
-                adam_moments_quantized(gr, kTable.v[256 * kTableMom + ((const uint8_t*)mom)[i]], sm, (float)((const uint8_t*)var)[i], sv, h, mn, vn);
-            } else {
-                adam_moments_plain(gr, load_elem<DT>(mom, i), load_elem<DT>(var, i), h, mn, vn);
-            }
-            float p;
-            if constexpr (EXACT) {
-                p = adam_apply_exact(DECOUPLED ? p0 * h.one_m_wd : p0, mn, vn, h);
-            } else {
-                float slack;
-                p = adam_apply_folded<DECOUPLED>(p0, mn, hw::sqrt(vn), h, AdamFoldedGuard<DT, ECCB>::value, slack);
-                if (adam_folded_is_flagged(slack)) {
-                    p = adam_apply_exact(DECOUPLED ? p0 * h.one_m_wd : p0, mn, vn, h);
-                    if (flagged) ++*flagged;
-                }
-            }
-            write_master<DT, ECCB>(param, ecc, i, p);
-            m[k] = mn; v[k] = vn;
-            am = fmaxf(am, fabsf(mn));
-            vmax = fmaxf(vmax, vn);
-        }
-        if (QUANT) {
-            // quick forms, each value verified and redone exactly if it fails (fo_math.h)
-            am = fmaxf(am, 1e-12f);
-            const float av_quick = fmaxf(hw::sqrt(vmax), 1e-12f);
-            const float av = fmaxf(sqrt_corrected(vmax), 1e-12f);
-            for (int k = 0; k < cnt; ++k) {
-                ((uint8_t*)mom)[g0 + k] = (uint8_t)quantize_mom_code_verified(m[k], am);
-                ((uint8_t*)var)[g0 + k] = (uint8_t)quantize_var_code_verified(v[k], av_quick, av);
-            }
-            mom_scales[group] = f32_to_f16(am);
-            var_scales[group] = f32_to_f16(av);
-        } else {
-            for (int k = 0; k < cnt; ++k) {
-                store_elem<DT>(mom, g0 + k, m[k]);
-                store_elem<DT>(var, g0 + k, v[k]);
-            }
+// ------------------------------------------------------------------------------------------------
+// a simulated wavefront: 64 lane states, the flows of fo_math.h run over it unchanged
+// ------------------------------------------------------------------------------------------------
+constexpr int kLanes = 64;
+
+struct FlowStats {   // what the flows did, for the tests
+    int64_t waves = 0;            // wavefronts stepped
+    int64_t questions = 0;        // wave.any() calls: one per flow and wavefront, plus one per position once a flow repairs
+    int64_t yes = 0;              // those answered with yes
+    int64_t codes_replaced = 0;   // set_*_code calls
+};
+FlowStats g_stats;
+
+template <class Lane> struct SimWave {
+    Lane* lanes;
+    template <class F> void each(F&& f) { for (int i = 0; i < kLanes; ++i) f(lanes[i]); }
+    // every lane evaluates the predicate (no short circuit), as under a ballot
+    template <class P> bool any(P&& p) {
+        bool r = false;
+        for (int i = 0; i < kLanes; ++i) r = p(const_cast<const Lane&>(lanes[i])) || r;
+        ++g_stats.questions;
+        g_stats.yes += r;
+        return r;
+    }
+};
+
+// lane states with the members the flows ask for; codes as plain integers (the kernels keep them packed)
+template <int N> struct MomLane {
+    float m[N], am = 1e-12f, x[N], slack[N], least = 0.0f, ram = 0.0f;
+    u32 code[N];
+    void convert_mom(const float (&q)[N]) { for (int k = 0; k < N; ++k) code[k] = (u32)hw::floor_to_int(q[k]) & 0xffu; }
+    void set_mom_code(int k, u32 c) { code[k] = c & 0xffu; ++g_stats.codes_replaced; }
+};
+template <int N> struct VarLane {
+    float v[N], r[N], av_quick = 1e-12f, av = 1e-12f, x[N], slack[N], least = 0.0f, rav = 0.0f;
+    u32 code[N];
+    void convert_var(const float (&q)[N]) { for (int k = 0; k < N; ++k) code[k] = (u32)(int)q[k] & 0xffu; }
+    void set_var_code(int k, u32 c) { code[k] = c & 0xffu; ++g_stats.codes_replaced; }
+};
+template <int N> struct BothLane {
+    float m[N], am = 1e-12f, v[N], r[N], av_quick = 1e-12f, av = 1e-12f;
+    float xm[N], xv[N], slack_m[N], slack_v[N], least_m = 0.0f, least_v = 0.0f, ram = 0.0f, rav = 0.0f;
+    u32 mcode[N], vcode[N];
+    void convert_both(const float (&qm)[N], const float (&qv)[N]) {
+        for (int k = 0; k < N; ++k) { mcode[k] = (u32)hw::floor_to_int(qm[k]) & 0xffu; vcode[k] = (u32)(int)qv[k] & 0xffu; }
+    }
+    void set_mom_code(int k, u32 c) { mcode[k] = c & 0xffu; ++g_stats.codes_replaced; }
+    void set_var_code(int k, u32 c) { vcode[k] = c & 0xffu; ++g_stats.codes_replaced; }
+};
+template <int N> struct RedoLane {
+    float p[N], slack[N], m[N], v[N], p_old[N], least = 0.0f;
+    float old_master(int k) const { return p_old[k]; }
+};
+
+// One moment's requantisation for a wavefront of lanes that hold N values each; lanes_per_group lanes share a
+// quantisation group.  m / v: kLanes * N values in lane order; live[l]: the lane owns at least one real element.
+// Writes the codes and (for lanes that lead a group) the fp16 scales.
+template <int N> void group_scales(const float* lane_am, const float* lane_vmax, float* am, float* av_quick, float* av) {
+    constexpr int per_group = kGroup / N;
+    for (int g0 = 0; g0 < kLanes; g0 += per_group) {
+        float a = 0.0f, vm = 0.0f;
+        for (int l = g0; l < g0 + per_group; ++l) { a = fmaxf(a, lane_am[l]); vm = fmaxf(vm, lane_vmax[l]); }
+        for (int l = g0; l < g0 + per_group; ++l) {
+            am[l] = fmaxf(a, 1e-12f);
+            av_quick[l] = fmaxf(hw::sqrt(vm), 1e-12f);
+            av[l] = fmaxf(sqrt_corrected(vm), 1e-12f);
         }
     }
 }
 
-// the structure of momentum_finish (fo_momentum.hip)
+// The structure of adam_finish (fo_adam.hip): one wavefront = kLanes lanes x EPL consecutive elements; lane l owns
+// elements [l * EPL, (l + 1) * EPL) of the span, elements past the end read as zero (scales as 1.0) and are never
+// stored.  `flagged` (may be null) counts the elements whose folded update was redone operation by operation.
+template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT>
+void adam_tensor(void* mom, uint16_t* mom_scales, void* var, uint16_t* var_scales, void* param, const void* grad, void* ecc,
+                 int64_t n, const AdamHyper& h, int64_t* flagged) {
+    constexpr int EPL = DTypeInfo<DT>::epl;
+    constexpr int kSpan = kLanes * EPL;
+    static RedoLane<EPL> redo[kLanes];
+    static MomLane<EPL> ml[kLanes];
+    static VarLane<EPL> vl[kLanes];
+    static BothLane<EPL> bl[kLanes];
+    for (int64_t base = 0; base < n; base += kSpan) {
+        ++g_stats.waves;
+        float lane_am[kLanes], lane_vmax[kLanes], r[kLanes][EPL];
+        for (int l = 0; l < kLanes; ++l) {
+            const int64_t first = base + (int64_t)l * EPL;
+            const bool live = first < n;
+            float sm = 1.0f, sv = 1.0f;                                       // masked scales read 1.0 (ref:2318-2323)
+            if (QUANT && live) { sm = f16_to_f32(mom_scales[first >> 5]); sv = f16_to_f32(var_scales[first >> 5]); }
+            lane_am[l] = lane_vmax[l] = 0.0f;
+            for (int k = 0; k < EPL; ++k) {
+                const int64_t i = first + k;
+                const bool in = i < n;
+                const float p0 = in ? read_master<DT, ECCB>(param, ecc, i) : 0.0f;
+                float gr = in ? load_elem<DT>(grad, i) : 0.0f;
+                if (!DECOUPLED) gr = gr + p0 * h.wd;
+                float mn, vn;
+                if (QUANT) {
+                    adam_moments_quantized(gr, kTable.v[256 * kTableMom + (in ? ((const uint8_t*)mom)[i] : 0)], sm,
+                                           in ? (float)((const uint8_t*)var)[i] : 0.0f, sv, h, mn, vn);
+                } else {
+                    adam_moments_plain(gr, in ? load_elem<DT>(mom, i) : 0.0f, in ? load_elem<DT>(var, i) : 0.0f, h, mn, vn);
+                }
+                const float rk = (QUANT || !EXACT) ? hw::sqrt(vn) : 0.0f;
+                RedoLane<EPL>& R = redo[l];
+                R.p_old[k] = p0; R.m[k] = mn; R.v[k] = vn; r[l][k] = rk;
+                if constexpr (EXACT) {
+                    R.p[k] = adam_apply_exact(DECOUPLED ? p0 * h.one_m_wd : p0, mn, vn, h);
+                    R.slack[k] = 0.0f;
+                } else {
+                    R.p[k] = adam_apply_folded<DECOUPLED>(p0, mn, rk, h, AdamFoldedGuard<DT, ECCB>::value, R.slack[k]);
+                    if (flagged && in && adam_folded_is_flagged(R.slack[k])) ++*flagged;
+                }
+                lane_am[l] = fmaxf(lane_am[l], fabsf(mn));
+                lane_vmax[l] = fmaxf(lane_vmax[l], vn);
+            }
+        }
+        if constexpr (!EXACT) {
+            SimWave<RedoLane<EPL>> wave{redo};
+            adam_redo_flagged<EPL, DECOUPLED>(wave, h);
+        }
+        for (int l = 0; l < kLanes; ++l)
+            for (int k = 0; k < EPL; ++k) {
+                const int64_t i = base + (int64_t)l * EPL + k;
+                if (i < n) write_master<DT, ECCB>(param, ecc, i, redo[l].p[k]);
+            }
+        if (QUANT) {
+            float am[kLanes], av_quick[kLanes], av[kLanes];
+            group_scales<EPL>(lane_am, lane_vmax, am, av_quick, av);
+            if constexpr (EPL == 8) {
+                for (int l = 0; l < kLanes; ++l) {
+                    ml[l].am = am[l]; vl[l].av_quick = av_quick[l]; vl[l].av = av[l];
+                    for (int k = 0; k < EPL; ++k) { ml[l].m[k] = redo[l].m[k]; vl[l].v[k] = redo[l].v[k]; vl[l].r[k] = r[l][k]; }
+                }
+                SimWave<MomLane<EPL>> mw{ml};
+                SimWave<VarLane<EPL>> vw{vl};
+                requantize_mom_verified<EPL>(mw);
+                requantize_var_verified<EPL>(vw);
+            } else {
+                for (int l = 0; l < kLanes; ++l) {
+                    bl[l].am = am[l]; bl[l].av_quick = av_quick[l]; bl[l].av = av[l];
+                    for (int k = 0; k < EPL; ++k) { bl[l].m[k] = redo[l].m[k]; bl[l].v[k] = redo[l].v[k]; bl[l].r[k] = r[l][k]; }
+                }
+                SimWave<BothLane<EPL>> bw{bl};
+                requantize_both_verified<EPL>(bw);
+            }
+            for (int l = 0; l < kLanes; ++l) {
+                const int64_t first = base + (int64_t)l * EPL;
+                for (int k = 0; k < EPL; ++k) {
+                    if (first + k >= n) break;
+                    ((uint8_t*)mom)[first + k] = (uint8_t)(EPL == 8 ? ml[l].code[k] : bl[l].mcode[k]);
+                    ((uint8_t*)var)[first + k] = (uint8_t)(EPL == 8 ? vl[l].code[k] : bl[l].vcode[k]);
+                }
+                if (first < n && (l & (kGroup / EPL - 1)) == 0) {                    // ref:2424-2434
+                    mom_scales[first >> 5] = f32_to_f16(am[l]);
+                    var_scales[first >> 5] = f32_to_f16(av[l]);
+                }
+            }
+        } else {
+            for (int l = 0; l < kLanes; ++l)
+                for (int k = 0; k < EPL; ++k) {
+                    const int64_t i = base + (int64_t)l * EPL + k;
+                    if (i < n) { store_elem<DT>(mom, i, redo[l].m[k]); store_elem<DT>(var, i, redo[l].v[k]); }
+                }
+        }
+    }
+}
+
+// the structure of momentum_finish (fo_momentum.hip), wavefront by wavefront
 template <int DT, int ECCB, bool QUANT, int KIND>
 void momentum_tensor(void* mom, uint16_t* mom_scales, void* param, const void* grad, void* ecc, int64_t n, const MomentumHyper& h) {
-    for (int64_t g0 = 0; g0 < n; g0 += kGroup) {
-        const int cnt = (int)((n - g0) < kGroup ? (n - g0) : kGroup);
-        const int64_t group = g0 >> 5;
-        float sm = 1.0f;
-        if (QUANT && KIND != KIND_PLAIN) sm = f16_to_f32(mom_scales[group]);
-        float m[kGroup];
-        float am = 0.0f;
-        for (int k = 0; k < cnt; ++k) {
-            const int64_t i = g0 + k;
-            float p = read_master<DT, ECCB>(param, ecc, i);
-            const float gr = load_elem<DT>(grad, i);
-            float mo = 0.0f;
-            if (KIND != KIND_PLAIN) mo = QUANT ? kTable.v[256 * kTableMom + ((const uint8_t*)mom)[i]] * sm : load_elem<DT>(mom, i);
-            momentum_element<KIND>(gr, p, mo, h, m[k]);
-            write_master<DT, ECCB>(param, ecc, i, p);
-            am = fmaxf(am, fabsf(m[k]));
+    constexpr int EPL = DTypeInfo<DT>::epl;
+    constexpr int kSpan = kLanes * EPL;
+    static MomLane<EPL> ml[kLanes];
+    for (int64_t base = 0; base < n; base += kSpan) {
+        ++g_stats.waves;
+        float lane_am[kLanes], lane_zero[kLanes];
+        for (int l = 0; l < kLanes; ++l) {
+            const int64_t first = base + (int64_t)l * EPL;
+            float sm = 1.0f;
+            if (QUANT && KIND != KIND_PLAIN && first < n) sm = f16_to_f32(mom_scales[first >> 5]);
+            lane_am[l] = lane_zero[l] = 0.0f;
+            for (int k = 0; k < EPL; ++k) {
+                const int64_t i = first + k;
+                const bool in = i < n;
+                float p = in ? read_master<DT, ECCB>(param, ecc, i) : 0.0f;
+                const float gr = in ? load_elem<DT>(grad, i) : 0.0f;
+                float mo = 0.0f;
+                if (KIND != KIND_PLAIN && in) mo = QUANT ? kTable.v[256 * kTableMom + ((const uint8_t*)mom)[i]] * sm : load_elem<DT>(mom, i);
+                momentum_element<KIND>(gr, p, mo, h, ml[l].m[k]);
+                if (in) write_master<DT, ECCB>(param, ecc, i, p);
+                lane_am[l] = fmaxf(lane_am[l], fabsf(ml[l].m[k]));
+            }
         }
         if (KIND == KIND_PLAIN) continue;
         if (QUANT) {
-            am = fmaxf(am, 1e-12f);
-            const float ram = hw::rcp(am);
-            for (int k = 0; k < cnt; ++k)  // as momentum_finish: 2-byte parameters go through the verified quick forms
-                ((uint8_t*)mom)[g0 + k] = (uint8_t)(DT == DT_F32 ? quantize_mom_code(m[k], am, ram) : quantize_mom_code_verified(m[k], am));
-            mom_scales[group] = f32_to_f16(am);
+            float am[kLanes], unused_q[kLanes], unused_e[kLanes];
+            group_scales<EPL>(lane_am, lane_zero, am, unused_q, unused_e);
+            for (int l = 0; l < kLanes; ++l) ml[l].am = am[l];
+            if constexpr (EPL == 8) {   // 2-byte parameters go through the verified quick forms
+                SimWave<MomLane<EPL>> mw{ml};
+                requantize_mom_verified<EPL>(mw);
+            } else {                    // fp32 parameters: the exact form on every value (fo_step.h: quantize_mom)
+                for (int l = 0; l < kLanes; ++l) {
+                    const float ram = hw::rcp(ml[l].am);
+                    for (int k = 0; k < EPL; ++k) ml[l].code[k] = quantize_mom_code(ml[l].m[k], ml[l].am, ram) & 0xffu;
+                }
+            }
+            for (int l = 0; l < kLanes; ++l) {
+                const int64_t first = base + (int64_t)l * EPL;
+                for (int k = 0; k < EPL && first + k < n; ++k) ((uint8_t*)mom)[first + k] = (uint8_t)ml[l].code[k];
+                if (first < n && (l & (kGroup / EPL - 1)) == 0) mom_scales[first >> 5] = f32_to_f16(am[l]);
+            }
         } else {
-            for (int k = 0; k < cnt; ++k) store_elem<DT>(mom, g0 + k, m[k]);
+            for (int l = 0; l < kLanes; ++l)
+                for (int k = 0; k < EPL; ++k) {
+                    const int64_t i = base + (int64_t)l * EPL + k;
+                    if (i < n) store_elem<DT>(mom, i, ml[l].m[k]);
+                }
         }
     }
 }
@@ -220,6 +352,40 @@ template <int DT, int EB, bool Q> struct MomentumRun {
 extern "C" {
 
 void hm_set_noise(int v) { fo_math_host_noise = v; }
+
+// Counters of the simulated wavefronts since the last reset: {waves, questions, yes, codes_replaced}.
+void hm_flow_stats(int64_t* out, int reset) {
+    out[0] = g_stats.waves; out[1] = g_stats.questions; out[2] = g_stats.yes; out[3] = g_stats.codes_replaced;
+    if (reset) g_stats = FlowStats();
+}
+
+// One wavefront (64 lanes x 8 values) through requantize_mom_verified / requantize_var_verified: m, v in lane order,
+// one group per 4 lanes.  The codes the flows deliver and, next to them, the exact forms' codes value by value.
+void hm_requantize_wave(const float* m, const float* v, uint8_t* qm, uint8_t* qv, uint8_t* qm_exact, uint8_t* qv_exact) {
+    static MomLane<8> ml[kLanes];
+    static VarLane<8> vl[kLanes];
+    float lane_am[kLanes], lane_vmax[kLanes], am[kLanes], av_quick[kLanes], av[kLanes];
+    for (int l = 0; l < kLanes; ++l) {
+        lane_am[l] = lane_vmax[l] = 0.0f;
+        for (int k = 0; k < 8; ++k) {
+            ml[l].m[k] = m[l * 8 + k]; vl[l].v[k] = v[l * 8 + k]; vl[l].r[k] = hw::sqrt(v[l * 8 + k]);
+            lane_am[l] = fmaxf(lane_am[l], fabsf(m[l * 8 + k])); lane_vmax[l] = fmaxf(lane_vmax[l], v[l * 8 + k]);
+        }
+    }
+    group_scales<8>(lane_am, lane_vmax, am, av_quick, av);
+    for (int l = 0; l < kLanes; ++l) { ml[l].am = am[l]; vl[l].av_quick = av_quick[l]; vl[l].av = av[l]; }
+    SimWave<MomLane<8>> mw{ml};
+    SimWave<VarLane<8>> vw{vl};
+    requantize_mom_verified<8>(mw);
+    requantize_var_verified<8>(vw);
+    for (int l = 0; l < kLanes; ++l)
+        for (int k = 0; k < 8; ++k) {
+            qm[l * 8 + k] = (uint8_t)ml[l].code[k];
+            qv[l * 8 + k] = (uint8_t)vl[l].code[k];
+            qm_exact[l * 8 + k] = (uint8_t)quantize_mom_code(m[l * 8 + k], am[l], hw::rcp(am[l]));
+            qv_exact[l * 8 + k] = (uint8_t)quantize_var_code(sqrt_corrected(v[l * 8 + k]), av[l], hw::rcp(av[l]));
+        }
+}
 
 // Arguments as fo_adam_step (include/flashoptim_hip.h) without the stream; host pointers.
 // exact: <= 0 = the choice the kernels make for this variant (fo_adam_step), 1 = operation by operation on every

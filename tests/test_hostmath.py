@@ -179,6 +179,89 @@ def test_quick_forms_with_verification_give_the_exact_requantisers_codes(noise):
     assert rate["continuous"] < 2e-3 and rate["first step"] > rate["continuous"]
 
 
+# ------------------------------------------------------------------------------------------------ wave-level flows
+
+
+def _centred_wave(seed):
+    """512 first-moment and 512 second-moment values (lane l holds values 8l .. 8l+7, four lanes per group) whose quick
+    pre-floor values sit in the middle between two integers: none fails the margin test."""
+    g = torch.Generator().manual_seed(seed)
+    m = torch.empty(16, 32, dtype=torch.float64)
+    v = torch.empty(16, 32, dtype=torch.float64)
+    for grp in range(16):
+        am = 10.0 ** float(torch.empty(1).uniform_(-6, 1, generator=g))
+        j = torch.randint(-126, 127, (32,), generator=g).double()
+        j[0] = 127.0                                       # the group's largest magnitude
+        t = j / 254.0                                      # x = 254 t + 0.5 = j + 0.5
+        m[grp] = am * t / (1.0 - t.abs())
+        av = 10.0 ** float(torch.empty(1).uniform_(-6, 1, generator=g))
+        jv = torch.randint(0, 255, (32,), generator=g).double()
+        jv[0] = 255.0
+        v[grp] = (av * jv / 255.0) ** 2                    # x = 255 r / av + 0.5 = jv + 0.5
+    return m.reshape(-1), v.reshape(-1)
+
+
+@pytest.mark.parametrize("noise", NOISE)
+def test_verified_flows_repair_exactly_the_lane_and_position_that_failed(noise):
+    """The control flow of the verified requantisation (fo_math.h: requantize_mom_verified, requantize_var_verified)
+    runs here over a simulated wavefront, the same text the kernels compile: a wavefront without a failing value
+    asks one question per flow and branches past the repair; one failing value in one lane makes the flow ask once per
+    element position, redo exactly that position and replace exactly that one code."""
+    H.set_noise(noise)
+    m, v = _centred_wave(3)
+    H.flow_stats()
+    qm, qv, em, ev = H.requantize_wave(m.float(), v.float())
+    assert torch.equal(qm, em) and torch.equal(qv, ev)
+    assert H.flow_stats() == dict(waves=0, questions=2, yes=0, codes_replaced=0)
+    for lane, pos, which in ((0, 1, "m"), (17, 5, "m"), (63, 7, "m"), (5, 3, "v"), (40, 1, "v"), (63, 6, "v")):
+        mm, vv = m.clone(), v.clone()
+        i, grp = lane * 8 + pos, (lane * 8 + pos) // 32
+        if which == "m":                                   # x = 254 t + 0.5 an integer: on the rounding boundary
+            am = float(mm[grp * 32:(grp + 1) * 32].abs().max())
+            t = (40.0 - 0.5) / 254.0
+            mm[i] = am * t / (1.0 - t)
+        else:
+            av = float(vv[grp * 32:(grp + 1) * 32].max()) ** 0.5
+            vv[i] = (av * (90.0 - 0.5) / 255.0) ** 2
+        qm, qv, em, ev = H.requantize_wave(mm.float(), vv.float())
+        assert torch.equal(qm, em) and torch.equal(qv, ev), (lane, pos, which)
+        st = H.flow_stats()
+        # the failing flow: one question for the wavefront, eight for the positions, two answered yes; the other: one
+        assert st == dict(waves=0, questions=1 + 8 + 1, yes=2, codes_replaced=1), (lane, pos, which, st)
+    # the same position failing in two lanes is still one position redone, two codes replaced
+    mm = m.clone()
+    for lane in (9, 50):
+        grp = lane * 8 // 32
+        am = float(mm[grp * 32:(grp + 1) * 32].abs().max())
+        t = (-30.0 - 0.5) / 254.0
+        mm[lane * 8 + 2] = am * t / (1.0 - abs(t))
+    qm, qv, em, ev = H.requantize_wave(mm.float(), v.float())
+    assert torch.equal(qm, em) and torch.equal(qv, ev)
+    assert H.flow_stats() == dict(waves=0, questions=10, yes=2, codes_replaced=2)
+
+
+@pytest.mark.parametrize("noise", [0, 7])
+def test_update_repair_flow_redoes_the_one_flagged_element(noise):
+    """adam_redo_flagged over simulated wavefronts: weights a thousand times larger than their updates except one, which
+    its update all but cancels.  That element alone is flagged, it comes out with the oracle's bits, and every other
+    element of its wavefront keeps its folded result (within one unit)."""
+    H.set_noise(noise)
+    n = 3 * 512 + 77
+    for where in (0, 700, 1535, n - 1):
+        a = _adam_state(n, torch.bfloat16, torch.int8, True, seed=8)
+        a["p"] = torch.full((n,), 1.5, dtype=torch.bfloat16)
+        g = _rand(n, 1e-3, 88).abs().add_(1e-4).to(torch.bfloat16)   # positive gradients: the first update is -lr
+        a["p"][where] = 1e-3 * (1.0 + 2.0 ** -7)                     # lands within a few 1e-6 of zero
+        b = _clone(a)
+        T.adam_step_ref(T.MomentState(b["m"], b["ms"]), T.MomentState(b["v"], b["vs"]), b["p"], g, b["e"], 1e-3, 0.9, 0.999, 1e-8, 0.0, True, 1)
+        flagged = H.adam_step(a["m"], a["ms"], a["v"], a["vs"], a["p"], g, a["e"], 1e-3, 0.9, 0.999, 1e-8, 0.0, True, 1)
+        assert flagged == 1, (where, flagged)
+        assert a["p"][where].view(torch.int16) == b["p"][where].view(torch.int16) and a["e"][where] == b["e"][where]
+        parity.check_master(a["p"], a["e"], b["p"], b["e"], f"one flagged element at {where}")
+        for key in ("m", "ms", "v", "vs"):
+            assert parity.bits_equal(a[key], b[key])
+
+
 # ------------------------------------------------------------------------------------------------ whole steps
 
 VARIANTS = [
