@@ -144,9 +144,14 @@ template <int DT, int ECCB, bool QUANT, bool DECOUPLED, bool EXACT = AdamExact<D
     //     (14: -4 points, 18 with five per SIMD: -5, 21 with six: -6; 16 without the cap per SIMD: -0.4);
     //   operation-by-operation update on 2-byte parameters (2-byte ECC, fp16 with a 1-byte ECC, the *_exact entry
     //     points): 20 with at most five per SIMD (16/4: -3.5 points, 18/5 and 21/6: -1.3, 25 and 32 uncapped: -3);
-    //   fp32 parameters (2.5 KiB of loads per wavefront): 18, no cap (a cap costs a point).
+    //   fp32 parameters (2.5 KiB of loads per wavefront), multi-tensor kernel: 21, with or without a cap of six or
+    //     seven per SIMD (18: -3.8 points, 25: -1.5, 32: -3; 20 with five per SIMD and 24 with six: -1); the
+    //     single-tensor kernel, launched tensor by tensor in gradient-release order (fewer registers, no launch
+    //     tables): 18 (21: -1.3 points, 25: -1.9).
     static constexpr bool kNarrowExact = EXACT && DT != DT_F32;
-    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 18 : (kNarrowExact ? 20 : 16);
+    static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 21 : (kNarrowExact ? 20 : 16);
+    static constexpr int kWorkgroupsPerCuShortTensors = kWorkgroupsPerCu;
+    static constexpr int kWorkgroupsPerCuSingleTensor = DT == DT_F32 ? 18 : kWorkgroupsPerCu;
     static constexpr int kMaxWavesPerSimd = DT == DT_F32 ? 8 : (kNarrowExact ? 5 : 4);
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
@@ -176,6 +181,8 @@ template <int DT, int ECCB, bool QUANT> struct AdamStreamsOp {
     // to four points slower), 14 with 2-byte ECC (16 one point slower); fp32 parameters (256 elements and 2.5 KiB per
     // wavefront, the codes as 4-byte loads) want every slot: 32 (79.6 %; 25: 79.2 %, 18: 74.6 %)
     static constexpr int kWorkgroupsPerCu = DT == DT_F32 ? 32 : (ECCB == 2 ? 14 : 16);
+    static constexpr int kWorkgroupsPerCuShortTensors = kWorkgroupsPerCu;
+    static constexpr int kWorkgroupsPerCuSingleTensor = kWorkgroupsPerCu;
     static constexpr int kMaxWavesPerSimd = 8;
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = AdamRaw<DT, ECCB, QUANT>;
@@ -319,7 +326,7 @@ static int multi_adam_step_any(const fo_tensor_desc* descs, int64_t n_tensors, c
     if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
     if (n_chunks == 0) return 0;
     if (step < 1) return fail(FO_ERR_INVALID_ARGUMENT, "step must be >= 1 (got %d)", step);
-    MultiLauncher<fo::AdamHyper> L{descs, chunks, n_chunks, make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step), (hipStream_t)stream};
+    MultiLauncher<fo::AdamHyper> L{descs, n_tensors, chunks, n_chunks, n_chunks, make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step), (hipStream_t)stream};
     return dispatch_adam(dtype, ecc_bytes, quantized, decoupled, exact, L);
 }
 
@@ -396,7 +403,7 @@ int fo_multi_adam_step_static(const fo_tensor_desc* host_descs, int64_t n_tensor
         hipLaunchKernelGGL(stage_tables_kernel, dim3((unsigned)b.count), dim3(256), 0, (hipStream_t)stream, b, d_descs, d_chunks);
         if (int rc = check_hip(hipGetLastError(), "table staging kernel launch")) return rc;
     }
-    MultiLauncher<fo::AdamHyper> L{d_descs, d_chunks, n_chunks, make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step), (hipStream_t)stream};
+    MultiLauncher<fo::AdamHyper> L{d_descs, n_tensors, d_chunks, n_chunks, total_tiles, make_adam_hyper(lr, beta1, beta2, eps, weight_decay, step), (hipStream_t)stream};
     return dispatch_adam(dtype, ecc_bytes, quantized, decoupled, 0, L);
 }
 
@@ -405,7 +412,7 @@ int fo_multi_adam_streams_copy(const fo_tensor_desc* descs, int64_t n_tensors, c
                                int dtype, int ecc_bytes, int quantized, void* stream) {
     if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
     if (n_chunks == 0) return 0;
-    MultiLauncher<fo::StreamsHyper> L{descs, chunks, n_chunks, fo::StreamsHyper{0u}, (hipStream_t)stream};
+    MultiLauncher<fo::StreamsHyper> L{descs, n_tensors, chunks, n_chunks, n_chunks, fo::StreamsHyper{0u}, (hipStream_t)stream};
     return dispatch<fo::AdamStreamsOp>(dtype, ecc_bytes, quantized, L);
 }
 

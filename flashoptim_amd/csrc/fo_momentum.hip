@@ -89,12 +89,16 @@ template <int DT, int ECCB, bool QUANT, int KIND> struct MomentumOp {
     using Hyper = MomentumHyper;
     static constexpr int kLutMask = ((QUANT && KIND != KIND_PLAIN) ? 1 << kTableMom : 0) | (ECCB == 1 ? 1 << kTableEcc : 0);  // LDS code tables
     static constexpr int kDtype = DT;
-    // measured on MI355X (3 KiB of loads per wavefront) over the residencies the LDS units allow (fo_step.h: 18, 21,
-    // 25, 32 around here): the 8B list is as fast at 21 as at 25, 4096 ragged tensors need 25 or more; capping the
-    // wavefronts per SIMD at 6 or 7 changes nothing measurable.
-    // (The ILP-oriented schedule that fo_adam.hip is built with gains 1-2 points on the 8B list at 18-21 resident
-    // workgroups and loses as much on the ragged list, which wants more than the 24 that its 80 VGPRs allow.)
-    static constexpr int kWorkgroupsPerCu = 25;
+    // Measured on MI355X (3 KiB of loads per wavefront) over the residencies the LDS units allow (fo_step.h: 18, 21,
+    // 25, 32 around here), Lion on bf16 parameters with a 1-byte ECC.  The 291 tensors of an 8B-parameter model: 21
+    // (82.5 % of the HBM peak; 18: 78.2, 25: 78.8, 32: 77.5).  4096 ragged tensors of 1e9 elements in all: 25 (80.9 %;
+    // 21: 79.9, 32: 80.5, 18: 77.6).  A launch therefore picks by the average length of its tensors
+    // (fo_step.h: is_short_tensor_list).  Capping the wavefronts per SIMD at 6 or 7 changes nothing measurable.
+    // (The ILP-oriented schedule that fo_adam.hip is built with would gain half a point on the ragged list at 21 and
+    // lose three on the 8B list.)
+    static constexpr int kWorkgroupsPerCu = 21;
+    static constexpr int kWorkgroupsPerCuShortTensors = 25;
+    static constexpr int kWorkgroupsPerCuSingleTensor = kWorkgroupsPerCu;
     static constexpr int kMaxWavesPerSimd = 8;
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = MomentumRaw<DT, ECCB, QUANT, KIND>;
@@ -121,6 +125,8 @@ template <int DT, int ECCB, bool QUANT> struct MomentumStreamsOp {
     // measured on MI355X: the 8B-parameter list streams fastest at 14 (83.2 %; 16: 82.0 %, 18: 79.6 %), 4096 ragged
     // tensors at 16 (81.8 %; 14: 80.2 %, 18: 81.5 %)
     static constexpr int kWorkgroupsPerCu = 16;
+    static constexpr int kWorkgroupsPerCuShortTensors = kWorkgroupsPerCu;
+    static constexpr int kWorkgroupsPerCuSingleTensor = kWorkgroupsPerCu;
     static constexpr int kMaxWavesPerSimd = 8;
     static constexpr int kEpl = DTypeInfo<DT>::epl;
     using Raw = MomentumRaw<DT, ECCB, QUANT, KIND_SGD>;
@@ -182,7 +188,7 @@ int fo_multi_momentum_step(const fo_tensor_desc* descs, int64_t n_tensors, const
                            float weight_decay, int decoupled, int nesterov, int do_lion, void* stream) {
     if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
     if (n_chunks == 0) return 0;
-    MultiLauncher<fo::MomentumHyper> L{descs, chunks, n_chunks, make_momentum_hyper(lr, mom_coef, update_coef, weight_decay, decoupled, nesterov), (hipStream_t)stream};
+    MultiLauncher<fo::MomentumHyper> L{descs, n_tensors, chunks, n_chunks, n_chunks, make_momentum_hyper(lr, mom_coef, update_coef, weight_decay, decoupled, nesterov), (hipStream_t)stream};
     return do_lion ? dispatch<LionOp>(dtype, ecc_bytes, quantized, L) : dispatch<SgdOp>(dtype, ecc_bytes, quantized, L);
 }
 
@@ -190,7 +196,7 @@ int fo_multi_sgd_plain_step(const fo_tensor_desc* descs, int64_t n_tensors, cons
                             int dtype, int ecc_bytes, float lr, float weight_decay, int decoupled, void* stream) {
     if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
     if (n_chunks == 0) return 0;
-    MultiLauncher<fo::MomentumHyper> L{descs, chunks, n_chunks, make_momentum_hyper(lr, 0.0f, 1.0f, weight_decay, decoupled, 0), (hipStream_t)stream};
+    MultiLauncher<fo::MomentumHyper> L{descs, n_tensors, chunks, n_chunks, n_chunks, make_momentum_hyper(lr, 0.0f, 1.0f, weight_decay, decoupled, 0), (hipStream_t)stream};
     return dispatch<PlainOp>(dtype, ecc_bytes, 0, L);
 }
 
@@ -199,7 +205,7 @@ int fo_multi_momentum_streams_copy(const fo_tensor_desc* descs, int64_t n_tensor
                                    int dtype, int ecc_bytes, int quantized, void* stream) {
     if (int rc = validate_multi(descs, n_tensors, chunks, n_chunks, dtype, ecc_bytes)) return rc;
     if (n_chunks == 0) return 0;
-    MultiLauncher<fo::MomentumStreamsHyper> L{descs, chunks, n_chunks, fo::MomentumStreamsHyper{0u}, (hipStream_t)stream};
+    MultiLauncher<fo::MomentumStreamsHyper> L{descs, n_tensors, chunks, n_chunks, n_chunks, fo::MomentumStreamsHyper{0u}, (hipStream_t)stream};
     return dispatch<fo::MomentumStreamsOp>(dtype, ecc_bytes, quantized, L);
 }
 

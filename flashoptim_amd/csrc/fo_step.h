@@ -364,19 +364,33 @@ Residency plan_residency(Kernel kernel, int target, int static_lds, int max_wave
     return r;
 }
 
-// Residency of kernel K for Op on the current device (planned at the first launch there).
-template <class Op, class Kernel> const Residency& residency_of(Kernel kernel) {
+// A kernel family may name a second residency for launches over many short tensors (Op::kWorkgroupsPerCuShortTensors):
+// every jump of the streams to another tensor's addresses costs machine time, and lists with thousands of such jumps
+// measured fastest with more wavefronts resident than a few long tensors want.  A launch counts as such when its
+// tensors average less than kShortTensorTiles tiles of 4096 elements.
+constexpr int64_t kShortTensorTiles = 256;
+inline bool is_short_tensor_list(int64_t n_tensors, int64_t n_tiles) { return n_tiles < kShortTensorTiles * n_tensors; }
+
+// The three launch shapes a kernel family may want different residencies for: the multi-tensor kernel over long
+// tensors (Op::kWorkgroupsPerCu), over many short tensors (Op::kWorkgroupsPerCuShortTensors), and the single-tensor
+// kernel (Op::kWorkgroupsPerCuSingleTensor).
+enum LaunchShape { kLongTensors = 0, kShortTensors = 1, kSingleTensor = 2 };
+
+// Residency of kernel K for Op on the current device (planned at the first launch of that shape there).
+template <class Op, class Kernel> const Residency& residency_of(Kernel kernel, LaunchShape shape) {
     constexpr int kMaxDevices = 64;
-    static Residency cache[kMaxDevices];
-    static std::once_flag once[kMaxDevices];
+    static Residency cache[kMaxDevices][3];
+    static std::once_flag once[kMaxDevices][3];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
-    std::call_once(once[dev], [&] {
+    std::call_once(once[dev][shape], [&] {
         const int forced = debug_workgroups_per_cu();
         constexpr int kStatic = fo::StepLut<Op::kLutMask>::kFloats * 4;
-        cache[dev] = plan_residency(kernel, forced > 0 ? forced : Op::kWorkgroupsPerCu, kStatic, Op::kMaxWavesPerSimd);
+        const int wanted = shape == kShortTensors ? Op::kWorkgroupsPerCuShortTensors
+                         : shape == kSingleTensor ? Op::kWorkgroupsPerCuSingleTensor : Op::kWorkgroupsPerCu;
+        cache[dev][shape] = plan_residency(kernel, forced > 0 ? forced : wanted, kStatic, Op::kMaxWavesPerSimd);
     });
-    return cache[dev];
+    return cache[dev][shape];
 }
 
 template <class Op>
@@ -384,16 +398,20 @@ int launch_single(const fo::TensorPtrs& t, const typename Op::Hyper& h, hipStrea
     // one pass over the tensor, one short-lived workgroup per span
     const int64_t grid = (t.n + fo::Span<Op>::kElems - 1) / fo::Span<Op>::kElems;
     if (grid > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "tensor too large for one launch (%lld elements)", (long long)t.n);
-    const unsigned lds = residency_of<Op>(fo::step_single_kernel<Op>).dynamic_lds;
+    const unsigned lds = residency_of<Op>(fo::step_single_kernel<Op>, kSingleTensor).dynamic_lds;
     hipLaunchKernelGGL(fo::step_single_kernel<Op>, dim3((unsigned)grid), dim3(fo::kBlockThreads), lds, stream, t, h);
     return check_hip(hipGetLastError(), "step kernel launch");
 }
 
+// n_tiles: 4096-element tiles the chunk table covers (n_chunks when a chunk is one tile; an estimate is good enough,
+// it only chooses between the two residencies)
 template <class Op>
-int launch_multi(const fo_tensor_desc* descs, const fo_chunk* chunks, int64_t n_chunks, const typename Op::Hyper& h, hipStream_t stream) {
+int launch_multi(const fo_tensor_desc* descs, int64_t n_tensors, const fo_chunk* chunks, int64_t n_chunks, int64_t n_tiles,
+                 const typename Op::Hyper& h, hipStream_t stream) {
     const int64_t grid = n_chunks * fo::Span<Op>::kPerTile;
     if (grid > INT32_MAX) return fail(FO_ERR_INVALID_ARGUMENT, "chunk table too large for one launch (%lld chunks)", (long long)n_chunks);
-    const unsigned lds = residency_of<Op>(fo::step_multi_kernel<Op>).dynamic_lds;
+    const LaunchShape shape = is_short_tensor_list(n_tensors, n_tiles) ? kShortTensors : kLongTensors;
+    const unsigned lds = residency_of<Op>(fo::step_multi_kernel<Op>, shape).dynamic_lds;
     hipLaunchKernelGGL(fo::step_multi_kernel<Op>, dim3((unsigned)grid), dim3(fo::kBlockThreads), lds, stream, descs, chunks, h);
     return check_hip(hipGetLastError(), "multi-tensor step kernel launch");
 }
@@ -415,9 +433,10 @@ int dispatch(int dtype, int ecc_bytes, int quantized, F&& f) {
 
 // Reports the residency plan of a kernel family (diagnostic entry points): 0 on success.
 struct ResidencyQuery {
-    int multi; int* target; int* achieved; int* dynamic_lds;
+    int multi; int* target; int* achieved; int* dynamic_lds;   // multi: 0 single-tensor kernel, 1 multi-tensor kernel, 2 the latter over short tensors
     template <class Op> int operator()() {
-        const Residency& r = multi ? residency_of<Op>(fo::step_multi_kernel<Op>) : residency_of<Op>(fo::step_single_kernel<Op>);
+        const Residency& r = multi ? residency_of<Op>(fo::step_multi_kernel<Op>, multi == 2 ? kShortTensors : kLongTensors)
+                                   : residency_of<Op>(fo::step_single_kernel<Op>, kSingleTensor);
         if (target) *target = r.target;
         if (achieved) *achieved = r.achieved;
         if (dynamic_lds) *dynamic_lds = (int)r.dynamic_lds;
@@ -430,8 +449,8 @@ template <class H> struct SingleLauncher {
     template <class Op> int operator()() { return launch_single<Op>(t, h, s); }
 };
 template <class H> struct MultiLauncher {
-    const fo_tensor_desc* d; const fo_chunk* c; int64_t nc; H h; hipStream_t s;
-    template <class Op> int operator()() { return launch_multi<Op>(d, c, nc, h, s); }
+    const fo_tensor_desc* d; int64_t nt; const fo_chunk* c; int64_t nc; int64_t tiles; H h; hipStream_t s;
+    template <class Op> int operator()() { return launch_multi<Op>(d, nt, c, nc, tiles, h, s); }
 };
 
 

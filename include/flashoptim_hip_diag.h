@@ -43,7 +43,8 @@ int fo_multi_momentum_streams_copy(const fo_tensor_desc *descs, int64_t n_tensor
  * for (`target`), what the dynamic LDS request that enforces it, the runtime's occupancy query and the kernel's cap
  * of wavefronts per SIMD allow together (`achieved`) and that request in bytes (`dynamic_lds`).  Any output pointer
  * may be NULL.
- *   multi: 0 = the single-tensor kernel, 1 = the multi-tensor kernel.
+ *   multi: 0 = the single-tensor kernel, 1 = the multi-tensor kernel, 2 = the multi-tensor kernel launched over a list
+ *          of many short tensors (the momentum kernels keep more wavefronts resident there).
  *   kind (momentum): 0 = SGD / SGDW / Nesterov, 1 = Lion, 2 = momentum-free SGD.
  */
 int fo_adam_step_residency(int dtype, int ecc_bytes, int quantized, int decoupled, int multi, int *target,

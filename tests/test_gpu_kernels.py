@@ -602,24 +602,26 @@ def test_randomised_configurations_match_oracle():
 def test_step_kernels_are_resident_as_planned():
     """Every step kernel bounds the workgroups resident on a compute unit by requesting unused LDS (streaming from
     HBM degrades with too many bytes in flight per compute unit), some also by capping the wavefronts per SIMD.  The
-    request is a whole number of the device's LDS allocation units; the runtime's occupancy query must confirm the
-    intended residency for every kernel family, in both grid shapes."""
+    request is a whole number of the device's LDS allocation units; the plan (LDS units, the runtime's occupancy
+    query and the cap per SIMD together) must give the intended residency for every kernel family, in both grid
+    shapes, and the second residency the momentum kernels keep for lists of many short tensors."""
     import ctypes
 
     lib = _diag_lib()  # the same sources and flags as the product library, plus the queries
-    want_adam = {(0, 0): 18, (1, 0): 16, (1, 1): 16, (1, 2): 20, (2, 0): 16, (2, 1): 20, (2, 2): 20}
-    for (dtype, ecc), want in want_adam.items():
+    want_adam = {(0, 0): 21, (1, 0): 16, (1, 1): 16, (1, 2): 20, (2, 0): 16, (2, 1): 20, (2, 2): 20}
+    for (dtype, ecc), want_multi in want_adam.items():
         for quantized in (1, 0):
-            for multi in (0, 1):
+            for multi in (0, 1, 2):
+                want = 18 if (dtype == 0 and multi == 0) else want_multi   # fp32: the single-tensor kernel wants fewer
                 t, a, lds = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
                 rc = lib.fo_adam_step_residency(dtype, ecc, quantized, 1, multi, ctypes.byref(t), ctypes.byref(a), ctypes.byref(lds))
                 assert rc == 0 and t.value == want and a.value == want, (dtype, ecc, quantized, multi, t.value, a.value, lds.value)
     for kind in (0, 1, 2):
         for (dtype, ecc) in want_adam:
-            for multi in (0, 1):
+            for multi, want in ((0, 21), (1, 21), (2, 25)):
                 t, a, lds = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
                 rc = lib.fo_momentum_step_residency(dtype, ecc, 1, kind, multi, ctypes.byref(t), ctypes.byref(a), ctypes.byref(lds))
-                assert rc == 0 and t.value == 25 and a.value == 25, (kind, dtype, ecc, multi, t.value, a.value, lds.value)
+                assert rc == 0 and t.value == want and a.value == want, (kind, dtype, ecc, multi, t.value, a.value, lds.value)
 
 
 def test_the_binding_shown_in_the_integration_notes_runs():
