@@ -22,7 +22,7 @@ from typing import Any, Callable, Literal, Optional, cast
 import torch
 import torch.nn as nn
 
-from . import kernels
+from . import _hostscan, kernels
 from .kernels import compute_ecc_bits, reconstruct_fp32_param
 from .launcher import BucketPlan, StepTensors
 from .state import QuantizedTensorSpec, _MaybeQuantizedTensor
@@ -491,6 +491,13 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
                         return False
                 continue
             plan, i = b.plan, 0
+            if _hostscan.scan is not None:
+                # the same walk in one C++ loop over the tensor objects (flashoptim_amd/hostscan)
+                found = _hostscan.scan(b.params, plan.table_address)
+                if found is None:
+                    return False
+                moved.extend((plan, j, ptr) for j, ptr in found)
+                continue
             for p, grad_ptr, param_ptr in zip(b.params, plan.grad_ptrs, plan.param_ptrs):
                 g = p.grad
                 if g is None or not p.requires_grad:
@@ -548,7 +555,8 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
                 and cache.epoch == self._plan_epoch
                 and cache.state_len == len(self.state)
                 and self._cached_numerics_ok(cache, group)
-                and cache.param_ids == list(map(id, group["params"]))
+                and (_hostscan.same_objects(cache.params, group["params"]) if _hostscan.same_objects is not None
+                     and type(group["params"]) is list else cache.param_ids == list(map(id, group["params"])))
                 and cache.signature == self._plan_signature(group)
                 and self._step_group_fast(cache, group)
             ):

@@ -128,6 +128,7 @@ class BucketPlan:
         self._keepalive = [(t.param, t.ecc, t.mom, t.mom_scales, t.var, t.var_scales) for t in tensors]
         self.grad_ptrs = [d.grad for d in self.table]
         self.param_ptrs = [d.param for d in self.table]
+        self.table_address = ctypes.addressof(self.table)  # for the C++ walk over the table (flashoptim_amd/_hostscan.py)
 
         if torch.cuda.is_current_stream_capturing():
             raise RuntimeError(

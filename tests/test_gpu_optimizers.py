@@ -748,10 +748,27 @@ def test_ecc_invariants_over_every_binade():
 # ------------------------------------------------------------------------------- cached step() plans
 
 
-def test_cached_step_plan_follows_moving_missing_and_freed_gradients():
+WALKS = ["c++", "python"]
+
+
+def _use_walk(monkeypatch, walk):
+    """The per-step check of a cached plan runs in C++ (flashoptim_amd/lib/_fo_hostscan.so) when that module is built
+    and in Python otherwise; both must behave alike."""
+    from flashoptim_amd import _hostscan
+
+    if walk == "c++":
+        assert _hostscan.scan is not None, "build it with make -C flashoptim_amd/hostscan"
+    else:
+        monkeypatch.setattr(_hostscan, "scan", None)
+        monkeypatch.setattr(_hostscan, "same_objects", None)
+
+
+@pytest.mark.parametrize("walk", WALKS)
+def test_cached_step_plan_follows_moving_missing_and_freed_gradients(walk, monkeypatch):
     """step() caches a group's launch tables after the first call.  The cache must notice gradients that were
     re-allocated at other addresses, fall back when a gradient is missing, never keep a freed gradient alive, and
     stay bit-identical to per-tensor stepping throughout."""
+    _use_walk(monkeypatch, walk)
     import gc
     import weakref
 
@@ -801,10 +818,12 @@ def _count_full_plans(opt):
     return calls
 
 
-def test_cached_step_plan_with_frozen_and_unused_parameters():
+@pytest.mark.parametrize("walk", WALKS)
+def test_cached_step_plan_with_frozen_and_unused_parameters(walk, monkeypatch):
     """A group that holds a frozen parameter and one that never receives a gradient (fine-tuning) still steps from
     the cached plan; the cache is dropped the moment the unused parameter gets a gradient, and the result stays
     bit-identical to per-tensor stepping."""
+    _use_walk(monkeypatch, walk)
     fo = _fo()
     shapes = [5000, 33, 4096, 70001, 0]
     pa, pb = _make_params(shapes, torch.bfloat16, 33), _make_params(shapes, torch.bfloat16, 33)
@@ -834,9 +853,11 @@ def test_cached_step_plan_with_frozen_and_unused_parameters():
     assert oa.state[pa[0]]["step"].item() == 6 and oa.state[pa[2]]["step"].item() == 2
 
 
-def test_cached_step_plan_notices_replaced_parameter_storage():
+@pytest.mark.parametrize("walk", WALKS)
+def test_cached_step_plan_notices_replaced_parameter_storage(walk, monkeypatch):
     """`p.data = ...` (what module.to() and friends do) moves a parameter to new memory; the cached launch table
     must not go on updating the old block."""
+    _use_walk(monkeypatch, walk)
     fo = _fo()
     shapes = [5000, 4096, 70001]
     pa, pb = _make_params(shapes, torch.bfloat16, 34), _make_params(shapes, torch.bfloat16, 34)

@@ -390,3 +390,50 @@ def test_packaging_declares_the_reference_entry_points():
     for target in points.values():
         module, _, name = target.partition(":")
         assert issubclass(getattr(importlib.import_module(module), name), torch.optim.Optimizer)
+
+
+# ------------------------------------------------------------------------------------------- host scan helper
+
+
+def test_hostscan_module_validates_a_launch_table_like_the_python_walk():
+    """flashoptim_amd/lib/_fo_hostscan.so (C++ over the tensor objects): the per-step check of a cached launch plan.
+    Unchanged tensors give an empty tuple; gradients that moved are reported with their new address; a missing,
+    frozen, strided, resized or re-typed gradient, a parameter on other storage or a non-tensor make it decline."""
+    from flashoptim_amd import _hostscan
+    from flashoptim_amd._native import FoTensorDesc
+
+    assert _hostscan.scan is not None, "build it with make -C flashoptim_amd/hostscan"
+    n = 50
+    params = [torch.nn.Parameter(torch.randn(10)) for _ in range(n)]
+    for p in params:
+        p.grad = torch.randn(10)
+    table = (FoTensorDesc * n)()
+    for d, p in zip(table, params):
+        d.param, d.grad, d.n = p.data_ptr(), p.grad.data_ptr(), 10
+    addr = ctypes.addressof(table)
+    assert _hostscan.scan(params, addr) == ()
+    keep = [p.grad for p in params]                        # keeps the old addresses from being handed out again
+    params[7].grad, params[9].grad = torch.randn(10), torch.randn(10)
+    assert _hostscan.scan(params, addr) == ((7, params[7].grad.data_ptr()), (9, params[9].grad.data_ptr()))
+    table[7].grad, table[9].grad = params[7].grad.data_ptr(), params[9].grad.data_ptr()
+    assert _hostscan.scan(params, addr) == ()
+
+    def declines(change, undo):
+        change()
+        got = _hostscan.scan(params, addr)
+        undo()
+        return got is None
+
+    p5, g5 = params[5], params[5].grad
+    assert declines(lambda: setattr(p5, "grad", None), lambda: setattr(p5, "grad", g5))
+    assert declines(lambda: setattr(p5, "grad", torch.randn(20)[::2]), lambda: setattr(p5, "grad", g5))
+    assert declines(lambda: setattr(p5, "grad", None) or p5.requires_grad_(False), lambda: (p5.requires_grad_(True), setattr(p5, "grad", g5)))
+    old = p5.data
+    assert declines(lambda: setattr(p5, "data", torch.randn(10)), lambda: setattr(p5, "data", old))
+    assert _hostscan.scan(params, addr) == ()
+    assert _hostscan.scan(params[:5] + [3], addr) is None
+    with pytest.raises(TypeError):
+        _hostscan.scan(tuple(params), addr)
+    assert _hostscan.same_objects(params, list(params)) and not _hostscan.same_objects(params, params[:-1])
+    assert not _hostscan.same_objects(params, params[1:] + params[:1])
+    del keep
