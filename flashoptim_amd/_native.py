@@ -88,6 +88,7 @@ DIAG_SIGNATURES = {
     "fo_multi_momentum_streams_copy": (_i32, [_vp, _i64, _vp, _i64, _i32, _i32, _i32, _vp]),
     "fo_adam_step_residency": (_i32, [_i32] * 5 + [_vp] * 3),
     "fo_momentum_step_residency": (_i32, [_i32] * 5 + [_vp] * 3),
+    "fo_probe_residency": (_i32, [_i32, _vp, _i64, _vp, _vp]),
 }
 
 

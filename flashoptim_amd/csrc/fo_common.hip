@@ -30,6 +30,31 @@ __global__ __launch_bounds__(kCopyThreads) void copy_kernel(u32x4* __restrict__ 
 }
 
 
+
+// Counts, per compute unit, how many workgroups of this kernel are resident at once: every one-wavefront workgroup
+// registers on its compute unit's counter (hardware id registers name the unit), lingers for a bounded number of
+// clock ticks so that the unit fills up, and signs off.  Launched with a given dynamic LDS size it shows how many
+// workgroups that size really admits, independent of what the runtime's occupancy query says.
+constexpr int kProbeSlots = 4096;  // 16 XCC ids x 8 shader engine ids x 32 (shader array, compute unit) ids
+__global__ __launch_bounds__(64) void residency_probe_kernel(unsigned* __restrict__ now, unsigned* __restrict__ most,
+                                                             long long linger_ticks) {
+    extern __shared__ unsigned char unused_lds[];
+    unsigned hw_id, xcc_id;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw_id));
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_id));
+    const unsigned cu = (hw_id >> 8) & 0x1fu, se = (hw_id >> 13) & 0x7u;  // cu_id with the shader array bit; se_id
+    const unsigned slot = ((xcc_id & 0xfu) * 8u + se) * 32u + cu;
+    if (threadIdx.x == 0) {
+        const unsigned mine = atomicAdd(&now[slot], 1u) + 1u;
+        atomicMax(&most[slot], mine);
+        const long long start = wall_clock64();
+        // bounded twice over (clock ticks and iterations): every wavefront leaves
+        for (int i = 0; i < 20000 && wall_clock64() - start < linger_ticks; ++i) __builtin_amdgcn_s_sleep(8);
+        atomicSub(&now[slot], 1u);
+    }
+    if (threadIdx.x == 4096) unused_lds[0] = 0;  // never true: keeps the dynamic allocation referenced
+}
+
 }  // namespace fo
 #endif  // FO_DIAG
 
@@ -145,6 +170,29 @@ int fo_copy_bytes(void* dst, const void* src, int64_t n_bytes, void* stream) {
     return check_hip(hipGetLastError(), "copy kernel launch");
 }
 
+
+int fo_probe_residency(int dynamic_lds_bytes, void* counters, int64_t counters_bytes, int* most_resident, void* stream) {
+    if (dynamic_lds_bytes < 0 || dynamic_lds_bytes > 65536) return fail(FO_ERR_INVALID_ARGUMENT, "dynamic_lds_bytes must be within 0 .. 65536");
+    if (!counters || counters_bytes < (int64_t)(2 * fo::kProbeSlots * sizeof(unsigned)))
+        return fail(FO_ERR_INVALID_ARGUMENT, "counters must hold %d bytes of device memory", (int)(2 * fo::kProbeSlots * sizeof(unsigned)));
+    if (!most_resident) return fail(FO_ERR_INVALID_ARGUMENT, "most_resident must not be NULL");
+    unsigned* now = static_cast<unsigned*>(counters);
+    unsigned* most = now + fo::kProbeSlots;
+    hipStream_t s = (hipStream_t)stream;
+    if (int rc = check_hip(hipMemsetAsync(now, 0, 2 * fo::kProbeSlots * sizeof(unsigned), s), "hipMemsetAsync")) return rc;
+    const int cus = compute_units();
+    if (cus <= 0) return fail(FO_ERR_NO_DEVICE, "no compute units reported");
+    // 64 workgroups per compute unit, each lingering 20 us of the 100 MHz wall clock: the units fill to their limit
+    hipLaunchKernelGGL(fo::residency_probe_kernel, dim3((unsigned)cus * 64u), dim3(64), (size_t)dynamic_lds_bytes, s, now, most, 2000LL);
+    if (int rc = check_hip(hipGetLastError(), "residency probe launch")) return rc;
+    static thread_local unsigned host[fo::kProbeSlots];
+    if (int rc = check_hip(hipMemcpyAsync(host, most, sizeof(host), hipMemcpyDeviceToHost, s), "hipMemcpyAsync")) return rc;
+    if (int rc = check_hip(hipStreamSynchronize(s), "hipStreamSynchronize")) return rc;
+    unsigned best = 0;
+    for (unsigned v : host) best = v > best ? v : best;
+    *most_resident = (int)best;
+    return 0;
+}
 #endif  // FO_DIAG
 
 }  // extern "C"

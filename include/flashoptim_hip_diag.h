@@ -52,6 +52,16 @@ int fo_adam_step_residency(int dtype, int ecc_bytes, int quantized, int decouple
 int fo_momentum_step_residency(int dtype, int ecc_bytes, int quantized, int kind, int multi, int *target,
                                int *achieved, int *dynamic_lds);
 
+/*
+ * Measures how many one-wavefront workgroups that request `dynamic_lds_bytes` of LDS a compute unit really holds at
+ * once: a probe kernel whose workgroups register on their compute unit (named by the hardware id registers), linger
+ * for 20 us and sign off; `most_resident` receives the largest count any unit reached.  The step kernels bound their
+ * residency through such requests (fo_adam_step_residency above reports the plan); this shows what the device makes
+ * of a request, independent of the runtime's occupancy query and of the allocation unit the plan assumes.
+ * `counters`: 32 KiB of device memory (scratch).  Synchronises the stream.
+ */
+int fo_probe_residency(int dynamic_lds_bytes, void *counters, int64_t counters_bytes, int *most_resident, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

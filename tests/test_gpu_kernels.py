@@ -624,6 +624,47 @@ def test_step_kernels_are_resident_as_planned():
                 assert rc == 0 and t.value == want and a.value == want, (kind, dtype, ecc, multi, t.value, a.value, lds.value)
 
 
+def test_lds_requests_admit_the_workgroups_the_residency_plan_assumes():
+    """The residency plan assumes that the device hands out LDS in units of 1280 bytes, 128 per compute unit, so that a
+    workgroup asking for k units leaves room for 128 // k workgroups.  Measured here, not assumed: a probe kernel
+    whose one-wavefront workgroups count themselves per compute unit is launched with requests of 4 .. 10 units (and
+    with one byte more than 4 and 8 units, which must cost a whole further unit), and the largest number resident
+    on any compute unit must be what the plan computes.  Then every step kernel's own request (the residency
+    queries) is put through the same probe: a workgroup of the probe needs fewer registers than any step kernel, so
+    the count it reaches is the bound the request enforces."""
+    import ctypes
+
+    lib = _diag_lib()
+    counters = torch.zeros(8192, dtype=torch.int32, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def resident(lds_bytes):
+        out = ctypes.c_int()
+        rc = lib.fo_probe_residency(lds_bytes, counters.data_ptr(), counters.numel() * 4, ctypes.byref(out), stream)
+        assert rc == 0, lib.fo_last_error()
+        return out.value
+
+    unit = 1280
+    for k in (4, 5, 6, 7, 8, 9, 10):
+        assert resident(k * unit) == 128 // k, f"{k} units"
+    assert resident(4 * unit + 1) == 128 // 5 and resident(8 * unit + 1) == 128 // 9
+    assert resident(0) == 32                       # eight wavefronts per SIMD, four SIMDs
+    seen = set()
+    for dtype, ecc in ((0, 0), (1, 0), (1, 1), (1, 2), (2, 1)):
+        for multi in (0, 1, 2):
+            for query, extra in ((lib.fo_adam_step_residency, (1,)), (lib.fo_momentum_step_residency, (1,))):
+                t, a, lds = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+                assert query(dtype, ecc, 1, *extra, multi, ctypes.byref(t), ctypes.byref(a), ctypes.byref(lds)) == 0
+                static = 2048 if ecc == 1 else 1024   # the kernels' own code tables come on top of the dynamic request
+                key = (lds.value + static, a.value)
+                if key in seen:
+                    continue
+                seen.add(key)
+                # the request enforces the planned residency, unless the kernel's cap per SIMD lowers it further
+                got = resident(lds.value + static)
+                assert got == a.value or (got > a.value and a.value % 4 == 0), (dtype, ecc, multi, lds.value, a.value, got)
+
+
 def test_the_binding_shown_in_the_integration_notes_runs():
     """The ctypes stub that the integration notes print (what a maintainer of the reference would add) is executed
     as written, against the built library, and gives the same bits as this package's own binding."""
