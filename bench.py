@@ -238,6 +238,17 @@ def build_workload(name: str, device):
                     desc="4096 bf16 tensors, lengths log-uniform in [1, 2^24], Student-t(3) gradients, "
                          + type(opt).__name__ + ", master_weight_bits=24",
                     launch="one multi-tensor launch per step", optimizer=type(opt).__name__, mwb=24)
+    if name == "llama8b-fp32":
+        shapes = llama3_8b_shapes()
+        g = torch.Generator().manual_seed(2)
+        scales = (10.0 ** (torch.rand(len(shapes), generator=g) * 2 - 1)).tolist()
+        params = make_params(shapes, torch.float32, device, scales)
+        opt = fo.FlashAdamW(params, master_weight_bits=None, **hp)
+        return dict(params=params, opt=opt, step=rotating_gradients(params, opt.step, device, scales, sets=2),
+                    bpp=bytes_per_param(4, 0, 2),
+                    desc="Llama-3-8B-shaped parameter list, fp32 parameters, FlashAdamW, quantised moments, gradients "
+                         "redrawn per step (2 rotating sets)",
+                    launch="one multi-tensor launch per step", optimizer="FlashAdamW", mwb=None)
     if name == "llama8b-fp32-release":
         shapes = llama3_8b_shapes()
         g = torch.Generator().manual_seed(2)
@@ -405,8 +416,9 @@ def measure(work, steps: int, warmup: int) -> dict:
 
 
 # The other configurations of the baseline, run after the default workload (a few steps each): the flat 2^30 tensor,
-# the 8B list with 32-bit masters, the 4096 ragged tensors under Lion and SGDW, the fp32 gradient-release order.
-SECONDARY = ("flat-2p30", "llama8b-mwb32", "ragged-lion", "ragged-sgdw", "llama8b-fp32-release")
+# the 8B list with 32-bit masters, the 4096 ragged tensors under Lion and SGDW, fp32 parameters in one launch and in
+# gradient-release order.
+SECONDARY = ("flat-2p30", "llama8b-mwb32", "ragged-lion", "ragged-sgdw", "llama8b-fp32", "llama8b-fp32-release")
 
 
 def run_secondary(name: str, device, steps: int, warmup: int, parity: bool) -> dict:
