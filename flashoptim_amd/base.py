@@ -493,7 +493,7 @@ class FlashOptimizer(torch.optim.Optimizer, abc.ABC):
             plan, i = b.plan, 0
             if _hostscan.scan is not None:
                 # the same walk in one C++ loop over the tensor objects (flashoptim_amd/hostscan)
-                found = _hostscan.scan(b.params, plan.table_address)
+                found = _hostscan.scan(b.params, plan.table_address, plan.n_tensors)
                 if found is None:
                     return False
                 moved.extend((plan, j, ptr) for j, ptr in found)

@@ -29,8 +29,6 @@ __global__ __launch_bounds__(kCopyThreads) void copy_kernel(u32x4* __restrict__ 
     }
 }
 
-
-
 // Counts, per compute unit, how many workgroups of this kernel are resident at once: every one-wavefront workgroup
 // registers on its compute unit's counter (hardware id registers name the unit), lingers for a bounded number of
 // clock ticks so that the unit fills up, and signs off.  Launched with a given dynamic LDS size it shows how many
@@ -169,7 +167,6 @@ int fo_copy_bytes(void* dst, const void* src, int64_t n_bytes, void* stream) {
                        (fo::u32x4*)dst, (const fo::u32x4*)src, n_vec, grid * fo::kCopyThreads, passes);
     return check_hip(hipGetLastError(), "copy kernel launch");
 }
-
 
 int fo_probe_residency(int dynamic_lds_bytes, void* counters, int64_t counters_bytes, int* most_resident, void* stream) {
     if (dynamic_lds_bytes < 0 || dynamic_lds_bytes > 65536) return fail(FO_ERR_INVALID_ARGUMENT, "dynamic_lds_bytes must be within 0 .. 65536");

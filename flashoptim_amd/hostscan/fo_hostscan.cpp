@@ -10,12 +10,15 @@
 // same_objects(a, b) -> bool
 //   whether the two lists hold the very same objects in the same order (the group's parameter list against the one the
 //   plan was built for).
-// scan(params, table_address) -> None | tuple of (index, new_gradient_address)
+// scan(params, table_address, table_entries) -> None | tuple of (index, new_gradient_address)
 //   params         list of the bucket's parameters, in table order
 //   table_address  address of the bucket's fo_tensor_desc array (host copy, include/flashoptim_hip.h)
+//   table_entries  its length; a list of another length is an error (ValueError)
 //   None: some parameter has no gradient, does not require one, moved to other storage, or its gradient changed
 //         dtype, device, size or contiguity -- the caller takes the full planning path.  Otherwise the gradients
 //         that now live at another address than the table says (empty tuple: the table is current).
+//         A tensor object that libtorch cannot answer these questions for (a wrapper subclass without storage)
+//         also gives None.
 #include <Python.h>
 
 #include <ATen/core/Tensor.h>
@@ -40,14 +43,20 @@ static_assert(sizeof(TensorDesc) == 64, "layout of fo_tensor_desc");
 PyObject* scan(PyObject*, PyObject* args) {
     PyObject* params = nullptr;
     unsigned long long address = 0;
-    if (!PyArg_ParseTuple(args, "OK", &params, &address)) return nullptr;
+    Py_ssize_t entries = 0;
+    if (!PyArg_ParseTuple(args, "OKn", &params, &address, &entries)) return nullptr;
     if (!PyList_CheckExact(params)) {
-        PyErr_SetString(PyExc_TypeError, "scan(params, table_address): params must be a list");
+        PyErr_SetString(PyExc_TypeError, "scan(params, table_address, table_entries): params must be a list");
         return nullptr;
     }
     const TensorDesc* table = reinterpret_cast<const TensorDesc*>(static_cast<uintptr_t>(address));
     const Py_ssize_t n = PyList_GET_SIZE(params);
+    if (n != entries || (n > 0 && table == nullptr)) {
+        PyErr_SetString(PyExc_ValueError, "scan: the parameter list and the launch table differ in length");
+        return nullptr;
+    }
     PyObject* moved = nullptr;
+    try {
     for (Py_ssize_t i = 0; i < n; ++i) {
         PyObject* obj = PyList_GET_ITEM(params, i);
         bool ok = THPVariable_Check(obj);
@@ -81,6 +90,10 @@ PyObject* scan(PyObject*, PyObject* args) {
             Py_RETURN_NONE;
         }
     }
+    } catch (...) {  // libtorch refused a query (e.g. data_ptr() of a tensor without storage): not a plan this walk can vouch for
+        Py_XDECREF(moved);
+        Py_RETURN_NONE;
+    }
     if (!moved) return PyTuple_New(0);
     PyObject* out = PyList_AsTuple(moved);
     Py_DECREF(moved);
@@ -103,7 +116,7 @@ PyObject* same_objects(PyObject*, PyObject* args) {
 
 PyMethodDef methods[] = {
     {"same_objects", same_objects, METH_VARARGS, "same_objects(a, b) -> bool: the same objects in the same order"},
-    {"scan", scan, METH_VARARGS, "scan(params, table_address) -> None | tuple of (index, gradient address)"},
+    {"scan", scan, METH_VARARGS, "scan(params, table_address, table_entries) -> None | tuple of (index, gradient address)"},
     {nullptr, nullptr, 0, nullptr},
 };
 

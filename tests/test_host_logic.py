@@ -398,7 +398,8 @@ def test_packaging_declares_the_reference_entry_points():
 def test_hostscan_module_validates_a_launch_table_like_the_python_walk():
     """flashoptim_amd/lib/_fo_hostscan.so (C++ over the tensor objects): the per-step check of a cached launch plan.
     Unchanged tensors give an empty tuple; gradients that moved are reported with their new address; a missing,
-    frozen, strided, resized or re-typed gradient, a parameter on other storage or a non-tensor make it decline."""
+    frozen, strided, resized or re-typed gradient, a parameter on other storage, a non-tensor or a tensor without
+    storage make it decline; a list of another length than the table is refused."""
     from flashoptim_amd import _hostscan
     from flashoptim_amd._native import FoTensorDesc
 
@@ -411,16 +412,16 @@ def test_hostscan_module_validates_a_launch_table_like_the_python_walk():
     for d, p in zip(table, params):
         d.param, d.grad, d.n = p.data_ptr(), p.grad.data_ptr(), 10
     addr = ctypes.addressof(table)
-    assert _hostscan.scan(params, addr) == ()
+    assert _hostscan.scan(params, addr, n) == ()
     keep = [p.grad for p in params]                        # keeps the old addresses from being handed out again
     params[7].grad, params[9].grad = torch.randn(10), torch.randn(10)
-    assert _hostscan.scan(params, addr) == ((7, params[7].grad.data_ptr()), (9, params[9].grad.data_ptr()))
+    assert _hostscan.scan(params, addr, n) == ((7, params[7].grad.data_ptr()), (9, params[9].grad.data_ptr()))
     table[7].grad, table[9].grad = params[7].grad.data_ptr(), params[9].grad.data_ptr()
-    assert _hostscan.scan(params, addr) == ()
+    assert _hostscan.scan(params, addr, n) == ()
 
     def declines(change, undo):
         change()
-        got = _hostscan.scan(params, addr)
+        got = _hostscan.scan(params, addr, n)
         undo()
         return got is None
 
@@ -430,10 +431,16 @@ def test_hostscan_module_validates_a_launch_table_like_the_python_walk():
     assert declines(lambda: setattr(p5, "grad", None) or p5.requires_grad_(False), lambda: (p5.requires_grad_(True), setattr(p5, "grad", g5)))
     old = p5.data
     assert declines(lambda: setattr(p5, "data", torch.randn(10)), lambda: setattr(p5, "data", old))
-    assert _hostscan.scan(params, addr) == ()
-    assert _hostscan.scan(params[:5] + [3], addr) is None
+    assert _hostscan.scan(params, addr, n) == ()
+    assert _hostscan.scan(params[:5] + [3], addr, 6) is None
     with pytest.raises(TypeError):
-        _hostscan.scan(tuple(params), addr)
+        _hostscan.scan(tuple(params), addr, n)
+    with pytest.raises(ValueError):                        # a list that is not the table's length is never walked
+        _hostscan.scan(params + params[:1], addr, n)
+    # a tensor object libtorch cannot give a data pointer for makes the walk decline instead of ending the process
+    meta = torch.nn.Parameter(torch.empty(10, device="meta"))
+    meta.grad = torch.empty(10, device="meta")
+    assert _hostscan.scan([meta], addr, 1) is None
     assert _hostscan.same_objects(params, list(params)) and not _hostscan.same_objects(params, params[:-1])
     assert not _hostscan.same_objects(params, params[1:] + params[:1])
     del keep
